@@ -129,6 +129,10 @@ def dense_attention(xq, keys, values, k_scaler=None, v_scaler=None, mask=None):
   """attention_kernel.py:605-633, in the input dtype like the reference."""
   xq, rep = reshape_heads(xq, keys)
   bsz, _, _, head_dim = xq.shape
+  if not keys.is_floating_point():
+    # int8 codes: the reference's einsum runs on jnp arrays, whose type
+    # promotion lifts the codes to the activation dtype (exact, |code| <= 128)
+    keys, values = keys.to(xq.dtype), values.to(xq.dtype)
   scores = torch.einsum("ikjl,ikml->ikjm", xq, keys) / math.sqrt(head_dim)
   if k_scaler is not None:
     scores = scores * _scale_view(k_scaler, bsz, keys.shape[2])
