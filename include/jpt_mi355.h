@@ -1,0 +1,295 @@
+/*
+ * jpt_mi355.h - C ABI of libjpt_mi355.so: the decode-time KV-cache path of
+ * jetstream-pytorch for AMD MI355X (gfx950).
+ *
+ * The reference has no foreign-function interface on this path: it is a
+ * Python API (jetstream_pt/cache_manager.py, page_attention_manager.py,
+ * attention_kernel.py).  Each entry point below names the reference function
+ * whose work it does; the Python package jetstream_pt_amd binds them with
+ * ctypes and keeps the reference's class and function signatures.
+ *
+ * Conventions
+ *   - every function returns an int32 status: JPT_OK or a negative JPT_E_*;
+ *     jpt_last_error() returns a thread-local message for the last failure;
+ *   - device pointers are plain `void*` into HBM owned by the caller; nothing
+ *     here allocates device memory; kernels write in place;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     calls only enqueue work, they never synchronise;
+ *   - all tensors are contiguous, row-major, with the shapes stated;
+ *   - dtype codes are JPT_BF16 / JPT_F32 / JPT_I8.
+ */
+#ifndef JPT_MI355_H_
+#define JPT_MI355_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define JPT_OK 0
+#define JPT_E_BADARG (-1)        /* -> ValueError  */
+#define JPT_E_NOPAGES (-2)       /* -> queue.Empty (free list exhausted) */
+#define JPT_E_PAGE_OVERFLOW (-3) /* -> IndexError  (max_pages_per_sequence) */
+#define JPT_E_HIP (-4)           /* -> RuntimeError */
+
+#define JPT_BF16 0
+#define JPT_F32 1
+#define JPT_I8 2
+
+#define JPT_ROUND_TRUNC 0 /* Int8KVCacheGenerate.quantize, cache_manager.py:532-537 */
+#define JPT_ROUND_RNE 1   /* quantize_tensor symmetric int8, quantize.py:58-75 */
+
+int32_t jpt_version(void);
+const char* jpt_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * KV line scatter: dst[l, b, h, pos[b], :] = src[l, b, h, 0, :]
+ *
+ * Replaces KVCacheGenerate.update eager branches (cache_manager.py:250-293),
+ * KVCacheGenerate.finalize / update_single_cache_line (:154-225) and
+ * Int8KVCacheGenerate.finalize / update_single_cache_line (:422-503,
+ * :584-657), which issue one scatter or one dynamic_update_slice per slot
+ * (and per layer) per tensor.  One launch writes up to JPT_MAX_LINE_TENSORS
+ * tensors (K, V and, for int8 caches, both scalers) for all layers.
+ *
+ * dst is (n_layers, batch, heads, seq, row_bytes) bytes, src is
+ * (n_layers, batch, heads, 1, row_bytes).  `pos` is an int32 device array of
+ * `pos_count` entries: batch (one position per slot) or 1 (ring buffer: one
+ * shared position).  A position outside [0, seq) writes nothing.
+ * ---------------------------------------------------------------------- */
+#define JPT_MAX_LINE_TENSORS 4
+typedef struct {
+  void* dst;
+  const void* src;
+  int32_t heads;
+  int32_t row_bytes;
+} jpt_line_tensor;
+
+int32_t jpt_kv_scatter_lines(const jpt_line_tensor* tensors, int32_t n_tensors,
+                             const int32_t* pos, int32_t pos_count,
+                             int32_t n_layers, int32_t batch, int32_t seq,
+                             void* stream);
+
+/* ------------------------------------------------------------------------
+ * Fused per-token absmax int8 quantisation + append.
+ *
+ * Replaces Int8KVCacheGenerate.quantize + .update (cache_manager.py:532-582):
+ * per token, absmax over (heads, dim) [or over dim when scale_heads == heads],
+ * scale and codes computed op by op in `scale_dtype` with the rounding rule
+ * `rounding`, codes written to out_* (the k_quant / kscale the reference
+ * returns, or its lazy stash new_ks[layer]) and, when cache_* is not NULL,
+ * scattered to cache[b, :, pos[b], :] and scale[b, :, pos[b]].
+ *
+ * new_k/new_v (batch, heads, 1, dim) in in_dtype (bf16 or f32);
+ * cache_k/cache_v (batch, heads, seq, dim) int8; k_scale/v_scale
+ * (batch, scale_heads, seq) scale_dtype; out_k/out_v (batch, heads, 1, dim)
+ * int8; out_k_scale/out_v_scale (batch, scale_heads) scale_dtype.  out_* may
+ * be NULL.  scale_dtype is in_dtype or JPT_F32.  An all-zero token yields
+ * scale 0 and codes 0 under JPT_ROUND_TRUNC.
+ * ---------------------------------------------------------------------- */
+typedef struct {
+  const void* new_k;
+  const void* new_v;
+  void* cache_k;
+  void* cache_v;
+  void* k_scale;
+  void* v_scale;
+  void* out_k;
+  void* out_v;
+  void* out_k_scale;
+  void* out_v_scale;
+  const int32_t* pos;
+  int32_t pos_count;
+  int32_t batch, heads, seq, dim;
+  int32_t in_dtype, scale_dtype, scale_heads, rounding;
+} jpt_quant_append_args;
+
+int32_t jpt_kv_append_quant_i8(const jpt_quant_append_args* args, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Paged KV cache.  Pages are (heads, total_pages, page_size, row_bytes).
+ *
+ * jpt_paged_insert   - PageAttentionManager.insert_prefill_cache
+ *   (page_attention_manager.py:83-142): src (heads, seq_len, row_bytes) is
+ *   split into pages; pages[h, page_ids[p], t, :] = src[h, p*ps + t, :], the
+ *   tail of the last page is zero-filled.  Two tensors (K, V) per launch.
+ * jpt_paged_append   - PageKVCacheGenerate.update (cache_manager.py:681-706):
+ *   for column j of `indices` (3, n_active) = (page, j*ps + tok, slot):
+ *   pages[h, page_j, tok_j, :] = src[slot_j, h, 0, :]; src is
+ *   (batch, heads, 1, row_bytes).
+ * jpt_paged_gather   - PageAttentionManager._compress_cache (:195-200):
+ *   dst[h, t, :] = pages[h, page_row[t / ps], t % ps, :] for t < length.
+ * `page_ids`, `indices`, `page_row` are int32 device arrays.
+ * ---------------------------------------------------------------------- */
+int32_t jpt_paged_insert(void* pages_k, void* pages_v, const void* src_k,
+                         const void* src_v, const int32_t* page_ids,
+                         int32_t n_pages, int32_t seq_len, int32_t heads,
+                         int32_t total_pages, int32_t page_size,
+                         int32_t row_bytes, void* stream);
+
+int32_t jpt_paged_append(void* pages_k, void* pages_v, const void* src_k,
+                         const void* src_v, const int32_t* indices,
+                         int32_t n_active, int32_t batch, int32_t heads,
+                         int32_t total_pages, int32_t page_size,
+                         int32_t row_bytes, void* stream);
+
+int32_t jpt_paged_gather(void* dst, const void* pages, const int32_t* page_row,
+                         int32_t length, int32_t heads, int32_t total_pages,
+                         int32_t page_size, int32_t row_bytes, void* stream);
+
+/* int8 pages (no reference counterpart: the reference's paged cache is
+ * bf16/f32 only, cache_manager.py:717-724).  Same row scatter as
+ * jpt_paged_append with the quantiser of jpt_kv_append_quant_i8 in front:
+ * codes to pages (heads, total_pages, page_size, dim) int8, scales to
+ * (scale_heads, total_pages, page_size) scale_dtype. */
+typedef struct {
+  const void* new_k;
+  const void* new_v;
+  void* pages_k;
+  void* pages_v;
+  void* k_scale_pages;
+  void* v_scale_pages;
+  const int32_t* indices; /* (3, n_active) */
+  int32_t n_active;
+  int32_t batch, heads, total_pages, page_size, dim;
+  int32_t in_dtype, scale_dtype, scale_heads, rounding;
+} jpt_paged_quant_append_args;
+
+int32_t jpt_paged_append_quant_i8(const jpt_paged_quant_append_args* args,
+                                  void* stream);
+
+/* ------------------------------------------------------------------------
+ * Decode attention.
+ *
+ * One argument block serves the three reference entry points:
+ *   jpt_attn_ragged - ragged_mha / ragged_mqa_reference
+ *     (attention_kernel.py:255-580): keys (batch, kv_heads, seq, dim),
+ *     positions < lengths[b] attended, returns o plus the running max and
+ *     softmax denominator.
+ *   jpt_attn_dense  - dense_attention / flash_attention (:605-710): all `seq`
+ *     positions (or < lengths[b] when given) plus an optional additive mask.
+ *   jpt_attn_paged  - call_paged_attention (:789-808): keys are pages
+ *     (kv_heads, total_pages, page_size, dim) addressed through page_table
+ *     (batch, max_pages); lengths required.
+ *
+ * q, out: (batch, q_heads, q_rows, dim) in q_dtype (bf16 or f32).  k, v in
+ * kv_dtype (bf16, f32 or int8).  k_scale/v_scale: NULL, or
+ * (batch, scale_heads, seq) [paged: (scale_heads, total_pages, page_size)]
+ * in scale_dtype; scores are multiplied by k_scale and probabilities by
+ * v_scale after the row sum, as the reference does (:303-315, :660-679).
+ * out_max/out_denom: NULL or float32 (batch, q_heads, q_rows): row max of
+ * the scaled scores (natural-log units) and the sum of exp(score - max).
+ * A row that attends nothing gives out = 0, max = -inf, denom = 0.
+ *
+ * mask: NULL or additive mask in mask_dtype, element
+ * (b, h, t, s) at mask + b*mask_stride_b + h*mask_stride_h + t*mask_stride_t + s
+ * (strides in elements; 0 broadcasts).
+ *
+ * new_k/new_v: NULL, or the step's new token (batch, kv_heads, 1, dim) in
+ * kv_dtype with new_k_scale/new_v_scale (batch, scale_heads) when
+ * quantised; it is attended as one more position and merged by
+ * log-sum-exp, which is what AttentionKernel / Int8KVAttentionKernel do in
+ * lazy-update mode with a second flash_attention call and seven elementwise
+ * ops (layers.py:534-550, :702-718).
+ *
+ * workspace: device scratch of at least jpt_attn_workspace_bytes(args)
+ * bytes, 256-byte aligned.  Its first JPT_ATTN_WS_STATE_BYTES must be zero
+ * before the first call and are left zero by every call; calls sharing one
+ * workspace must not overlap in time.
+ * ---------------------------------------------------------------------- */
+#define JPT_ATTN_WS_STATE_BYTES 65536
+
+typedef struct {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* k_scale;
+  const void* v_scale;
+  const int32_t* lengths;
+  const int32_t* page_table;
+  const void* mask;
+  const void* new_k;
+  const void* new_v;
+  const void* new_k_scale;
+  const void* new_v_scale;
+  void* out;
+  float* out_max;
+  float* out_denom;
+  void* workspace;
+  int64_t workspace_bytes;
+  int64_t mask_stride_b, mask_stride_h, mask_stride_t;
+  int32_t batch, q_heads, kv_heads, q_rows, dim;
+  int32_t seq;         /* dense/ragged: cache length; paged: ignored */
+  int32_t total_pages; /* paged only */
+  int32_t page_size;   /* paged only */
+  int32_t max_pages;   /* paged only: row length of page_table */
+  int32_t q_dtype, kv_dtype, scale_dtype, scale_heads, mask_dtype;
+  float sm_scale;      /* multiplies q.k; 1/sqrt(dim) for ragged/dense/flash */
+  int32_t force_generic; /* 1 = use the shape-generic kernel (testing aid) */
+  int32_t reuse_plan;    /* 1 = the workspace already holds the split plan for
+                            these lengths (same batch, heads and lengths as the
+                            previous call on this workspace): skip planning.
+                            A decode step plans once and reuses it per layer. */
+} jpt_attn_args;
+
+int64_t jpt_attn_workspace_bytes(const jpt_attn_args* args);
+/* Plans the split of every slot's positions into workgroup-sized chunks and
+ * stores the plan in args->workspace without running attention; later calls
+ * on that workspace with reuse_plan = 1 skip planning.  Only lengths,
+ * batch, q_heads, kv_heads, q_rows, seq (or max_pages and page_size when
+ * `paged` is non-zero) and the workspace fields are read.  The reference
+ * computes its per-step block tables the same way, once per decode step for
+ * all layers (precompute_ragged_block_indices, engine.py:674-729). */
+int32_t jpt_attn_plan(const jpt_attn_args* args, int32_t paged, void* stream);
+int32_t jpt_attn_ragged(const jpt_attn_args* args, void* stream);
+int32_t jpt_attn_dense(const jpt_attn_args* args, void* stream);
+int32_t jpt_attn_paged(const jpt_attn_args* args, void* stream);
+
+/* Log-sum-exp merge of two partial attention results (layers.py:539-548):
+ * out = (l1*a*o1 + b*o2*l2) / (a*l1 + b*l2), a = exp(m1-g), b = exp(m2-g),
+ * g = max(m1, m2).  o*: (rows, dim) in dtype; m*, l*: float32 (rows). */
+int32_t jpt_lse_merge(void* out, const void* o1, const float* m1,
+                      const float* l1, const void* o2, const float* m2,
+                      const float* l2, int64_t rows, int32_t dim,
+                      int32_t dtype, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Host page allocator: PageAttentionManager (page_attention_manager.py:21-64,
+ * :145-177, :214-222).  FIFO free list, page table (batch, max_pages) int32
+ * initialised to the sentinel total_pages-1, lengths (batch) int32.  The
+ * tables live in host memory owned by the handle; jpt_pam_tables exposes
+ * them (valid until jpt_pam_destroy).  `free_order` is NULL (pages are
+ * handed out 0, 1, 2, ... as in the reference) or total_pages page ids.
+ * All methods take one internal mutex.
+ * ---------------------------------------------------------------------- */
+typedef struct jpt_pam jpt_pam;
+
+int32_t jpt_pam_create(int32_t batch, int32_t total_pages, int32_t page_size,
+                       int32_t max_pages, const int32_t* free_order,
+                       jpt_pam** out);
+void jpt_pam_destroy(jpt_pam* pam);
+int32_t jpt_pam_tables(jpt_pam* pam, int32_t** page_indices, int32_t** lengths);
+/* reserve_pages_insert: sets lengths[slot], pops ceil(seq_len/ps) pages into
+ * the row; *num_pages receives the count. */
+int32_t jpt_pam_reserve_insert(jpt_pam* pam, int32_t slot, int32_t seq_len,
+                               int32_t* num_pages);
+/* reserve_pages_decode: pops one page when seq_len > 0 sits on a boundary. */
+int32_t jpt_pam_reserve_decode(jpt_pam* pam, int32_t slot, int32_t seq_len);
+/* fill_new_pages: reserve_pages_decode for every slot in ascending order. */
+int32_t jpt_pam_fill_new_pages(jpt_pam* pam, const int32_t* lens);
+/* get_page_token_indices: writes (3, n_active) row-major into out (capacity
+ * 3*batch), sets *n_active, and lengths = lens == 0 ? 0 : lens + 1. */
+int32_t jpt_pam_page_token_indices(jpt_pam* pam, const int32_t* lens,
+                                   int32_t* out, int32_t* n_active);
+/* free_pages_resource: returns the slot's pages to the tail of the free
+ * list in row order, resets the row to the sentinel and the length to 0. */
+int32_t jpt_pam_free(jpt_pam* pam, int32_t slot);
+/* number of pages on the free list; with out != NULL (capacity total_pages)
+ * also copies the list in FIFO order. */
+int32_t jpt_pam_free_count(jpt_pam* pam, int32_t* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* JPT_MI355_H_ */

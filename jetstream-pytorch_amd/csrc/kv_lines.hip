@@ -1,0 +1,275 @@
+// Per-slot KV line writes: plain scatter (bf16/f32/int8 caches and scalers,
+// one or all layers) and the fused per-token absmax int8 quantiser + scatter.
+//
+// Both are pure data movement bound by HBM bandwidth and, at decode sizes
+// (one token per slot), by launch latency: one launch covers K and V (and
+// both scalers) for every layer.
+#include "common.h"
+
+namespace jpt {
+namespace {
+
+struct LineParams {
+  jpt_line_tensor t[JPT_MAX_LINE_TENSORS];
+  int32_t vec[JPT_MAX_LINE_TENSORS];  // bytes one thread moves, per tensor
+  const int32_t* pos;
+  int32_t pos_count, n_layers, batch, seq;
+};
+
+template <typename V>
+__device__ __forceinline__ void copy_vec(void* dst, const void* src, int v) {
+  static_cast<V*>(dst)[v] = static_cast<const V*>(src)[v];
+}
+
+// grid.y = tensor; a thread moves one vector of one (layer, slot, head) line.
+__global__ void __launch_bounds__(256) scatter_lines_kernel(LineParams p) {
+  const jpt_line_tensor t = p.t[blockIdx.y];
+  const int vec = p.vec[blockIdx.y];
+  const int vec_per_row = t.row_bytes / vec;
+  const int64_t total = static_cast<int64_t>(p.n_layers) * p.batch * t.heads * vec_per_row;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int v = static_cast<int>(i % vec_per_row);
+    const int64_t line = i / vec_per_row;  // (layer, slot, head)
+    const int h = static_cast<int>(line % t.heads);
+    const int64_t lb = line / t.heads;
+    const int b = static_cast<int>(lb % p.batch);
+    const int at = p.pos[p.pos_count == 1 ? 0 : b];
+    if (at < 0 || at >= p.seq) continue;
+    const char* src = static_cast<const char*>(t.src) + line * t.row_bytes;
+    char* dst = static_cast<char*>(t.dst) + ((lb * t.heads + h) * p.seq + at) * t.row_bytes;
+    switch (vec) {
+      case 16: copy_vec<uint4>(dst, src, v); break;
+      case 8: copy_vec<uint2>(dst, src, v); break;
+      case 4: copy_vec<uint32_t>(dst, src, v); break;
+      case 2: copy_vec<uint16_t>(dst, src, v); break;
+      default: copy_vec<uint8_t>(dst, src, v); break;
+    }
+  }
+}
+
+// Widest power-of-two vector (<= 16 bytes) that divides the row and matches
+// both base pointers.
+int vector_bytes(const jpt_line_tensor& t) {
+  for (int v = 16; v > 1; v >>= 1)
+    if (t.row_bytes % v == 0 && aligned(t.dst, v) && aligned(t.src, v)) return v;
+  return 1;
+}
+
+// ---- fused quantiser -------------------------------------------------------
+
+struct QuantParams {
+  jpt_quant_append_args a;
+  // paged destination (jpt_paged_append_quant_i8): rows are addressed through
+  // `indices` (3, n_active) instead of pos
+  const int32_t* indices;
+  int32_t n_active, total_pages, page_size;
+};
+
+template <bool ROUND_BF16>
+__device__ __forceinline__ float rnd(float x) {
+  return ROUND_BF16 ? round_to_bf16(x) : x;
+}
+
+// One workgroup per (token, tensor): blockIdx.x = token (slot, or active
+// index j when paged), blockIdx.y = 0 for K, 1 for V.  The op order is the
+// reference's, each op rounded to the scale dtype:
+//   trunc: a = absmax; s = a / 127;             q = x / s;      code = trunc(q)
+//   rne:   a = max(absmax, eps); s = a / 127; r = 1 / s; q = x * r;
+//          code = clamp(rint(q), -128, 127)
+template <bool BF16_MATH>
+__global__ void __launch_bounds__(256) quant_append_kernel(QuantParams p) {
+  const jpt_quant_append_args& a = p.a;
+  const bool paged = p.indices != nullptr;
+  const int tok = blockIdx.x;
+  const int b = paged ? p.indices[2 * p.n_active + tok] : tok;
+  const bool is_v = blockIdx.y == 1;
+  const void* src = is_v ? a.new_v : a.new_k;
+  int8_t* cache = static_cast<int8_t*>(is_v ? a.cache_v : a.cache_k);
+  void* scale_out = is_v ? a.v_scale : a.k_scale;
+  int8_t* stash = static_cast<int8_t*>(is_v ? a.out_v : a.out_k);
+  void* stash_scale = is_v ? a.out_v_scale : a.out_k_scale;
+
+  const int H = a.heads, D = a.dim, HD = H * D;
+  const int groups = a.scale_heads;           // 1 or H
+  const int per_group = HD / groups;          // elements sharing one scale
+  const int64_t src_base = static_cast<int64_t>(b) * HD;
+
+  __shared__ float s_red[4];
+  __shared__ float s_scale[64 + 1];  // per group (heads <= 64 when per-head)
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+  for (int g = 0; g < groups; ++g) {
+    float m = 0.f;
+    for (int i = threadIdx.x; i < per_group; i += blockDim.x)
+      m = fmaxf(m, fabsf(load_as_f32(src, src_base + g * per_group + i, a.in_dtype)));
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    if (lane == 0) s_red[wave] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float amax = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+      if (a.rounding == JPT_ROUND_RNE) amax = fmaxf(amax, rnd<BF16_MATH>(1e-5f));
+      s_scale[g] = rnd<BF16_MATH>(amax / 127.0f);
+    }
+    __syncthreads();
+  }
+
+  // destination of this token's rows
+  int at, page = 0;
+  bool write_cache = cache != nullptr;
+  if (paged) {
+    page = p.indices[tok];
+    at = p.indices[p.n_active + tok] % p.page_size;
+    write_cache = write_cache && page >= 0 && page < p.total_pages;
+  } else {
+    at = a.pos ? a.pos[a.pos_count == 1 ? 0 : b] : 0;
+    write_cache = write_cache && at >= 0 && at < a.seq;
+  }
+
+  for (int i = threadIdx.x; i < HD; i += blockDim.x) {
+    const int h = i / D, d = i - h * D;
+    const float s = s_scale[groups == 1 ? 0 : h];
+    const float x = load_as_f32(src, src_base + i, a.in_dtype);
+    int code;
+    if (a.rounding == JPT_ROUND_TRUNC) {
+      const float q = rnd<BF16_MATH>(x / s);
+      code = (q != q) ? 0 : static_cast<int>(q);  // 0/0 -> 0; cast truncates
+    } else {
+      const float r = rnd<BF16_MATH>(1.0f / s);
+      const float q = rnd<BF16_MATH>(x * r);
+      code = static_cast<int>(fminf(fmaxf(rintf(q), -128.f), 127.f));
+    }
+    const int8_t c = static_cast<int8_t>(code);
+    if (stash) stash[src_base + i] = c;
+    if (write_cache) {
+      const int64_t row = paged
+          ? (static_cast<int64_t>(h) * p.total_pages + page) * p.page_size + at
+          : (static_cast<int64_t>(b) * H + h) * a.seq + at;
+      cache[row * D + d] = c;
+    }
+  }
+  if (threadIdx.x < groups) {
+    const int g = threadIdx.x;
+    const float s = s_scale[g];
+    if (stash_scale) store_from_f32(stash_scale, static_cast<int64_t>(b) * groups + g, a.scale_dtype, s);
+    if (write_cache && scale_out) {
+      const int64_t idx = paged
+          ? (static_cast<int64_t>(g) * p.total_pages + page) * p.page_size + at
+          : (static_cast<int64_t>(b) * groups + g) * a.seq + at;
+      store_from_f32(scale_out, idx, a.scale_dtype, s);
+    }
+  }
+}
+
+int32_t check_quant_common(int32_t heads, int32_t dim, int32_t in_dtype,
+                           int32_t scale_dtype, int32_t scale_heads,
+                           int32_t rounding) {
+  JPT_REQUIRE(heads > 0 && dim > 0, "heads and dim must be positive");
+  JPT_REQUIRE(in_dtype == JPT_BF16 || in_dtype == JPT_F32, "in_dtype must be bf16 or f32");
+  JPT_REQUIRE(scale_dtype == in_dtype || scale_dtype == JPT_F32,
+              "scale_dtype must equal in_dtype or be f32");
+  JPT_REQUIRE(scale_heads == 1 || scale_heads == heads, "scale_heads must be 1 or heads");
+  JPT_REQUIRE(scale_heads <= 64, "per-head scales support at most 64 heads");
+  JPT_REQUIRE(rounding == JPT_ROUND_TRUNC || rounding == JPT_ROUND_RNE, "bad rounding mode");
+  return JPT_OK;
+}
+
+int32_t launch_quant(const QuantParams& p, int32_t tokens, hipStream_t stream) {
+  if (tokens == 0) return JPT_OK;
+  dim3 grid(tokens, 2);
+  if (p.a.scale_dtype == JPT_BF16)
+    hipLaunchKernelGGL(quant_append_kernel<true>, grid, dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL(quant_append_kernel<false>, grid, dim3(256), 0, stream, p);
+  return launch_status("quant_append_kernel");
+}
+
+}  // namespace
+}  // namespace jpt
+
+extern "C" {
+
+int32_t jpt_kv_scatter_lines(const jpt_line_tensor* tensors, int32_t n_tensors,
+                             const int32_t* pos, int32_t pos_count,
+                             int32_t n_layers, int32_t batch, int32_t seq,
+                             void* stream) {
+  using namespace jpt;
+  JPT_REQUIRE(tensors != nullptr && pos != nullptr, "NULL argument");
+  JPT_REQUIRE(n_tensors >= 1 && n_tensors <= JPT_MAX_LINE_TENSORS, "n_tensors must be 1..%d", JPT_MAX_LINE_TENSORS);
+  JPT_REQUIRE(n_layers > 0 && batch > 0 && seq > 0, "n_layers, batch, seq must be positive");
+  JPT_REQUIRE(pos_count == 1 || pos_count == batch, "pos_count must be 1 or batch");
+  LineParams p{};
+  int64_t most = 0;
+  for (int i = 0; i < n_tensors; ++i) {
+    JPT_REQUIRE(tensors[i].dst && tensors[i].src, "tensor %d has a NULL pointer", i);
+    JPT_REQUIRE(tensors[i].heads > 0 && tensors[i].row_bytes > 0, "tensor %d: heads and row_bytes must be positive", i);
+    p.t[i] = tensors[i];
+    p.vec[i] = vector_bytes(tensors[i]);
+    const int64_t n = static_cast<int64_t>(n_layers) * batch * tensors[i].heads * (tensors[i].row_bytes / p.vec[i]);
+    most = n > most ? n : most;
+  }
+  p.pos = pos;
+  p.pos_count = pos_count;
+  p.n_layers = n_layers;
+  p.batch = batch;
+  p.seq = seq;
+  int64_t blocks = (most + 255) / 256;
+  if (blocks > 65535) blocks = 65535;
+  dim3 grid(static_cast<unsigned>(blocks), n_tensors);
+  hipLaunchKernelGGL(scatter_lines_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), p);
+  return launch_status("scatter_lines_kernel");
+}
+
+int32_t jpt_kv_append_quant_i8(const jpt_quant_append_args* args, void* stream) {
+  using namespace jpt;
+  JPT_REQUIRE(args != nullptr, "args is NULL");
+  const jpt_quant_append_args& a = *args;
+  JPT_REQUIRE(a.new_k && a.new_v, "new_k/new_v are NULL");
+  JPT_REQUIRE(a.batch > 0, "batch must be positive");
+  int32_t st = check_quant_common(a.heads, a.dim, a.in_dtype, a.scale_dtype, a.scale_heads, a.rounding);
+  if (st != JPT_OK) return st;
+  const bool to_cache = a.cache_k != nullptr || a.cache_v != nullptr;
+  if (to_cache) {
+    JPT_REQUIRE(a.cache_k && a.cache_v && a.k_scale && a.v_scale, "cache_k, cache_v, k_scale, v_scale must all be set");
+    JPT_REQUIRE(a.pos != nullptr && (a.pos_count == 1 || a.pos_count == a.batch), "pos must hold 1 or batch entries");
+    JPT_REQUIRE(a.seq > 0, "seq must be positive");
+  } else {
+    JPT_REQUIRE(a.out_k && a.out_v && a.out_k_scale && a.out_v_scale, "nothing to write: cache_* and out_* are NULL");
+  }
+  QuantParams p{};
+  p.a = a;
+  return launch_quant(p, a.batch, static_cast<hipStream_t>(stream));
+}
+
+int32_t jpt_paged_append_quant_i8(const jpt_paged_quant_append_args* args, void* stream) {
+  using namespace jpt;
+  JPT_REQUIRE(args != nullptr, "args is NULL");
+  const jpt_paged_quant_append_args& g = *args;
+  JPT_REQUIRE(g.new_k && g.new_v && g.pages_k && g.pages_v && g.k_scale_pages && g.v_scale_pages, "NULL tensor argument");
+  JPT_REQUIRE(g.n_active >= 0 && g.n_active <= g.batch, "n_active must be 0..batch");
+  JPT_REQUIRE(g.n_active == 0 || g.indices != nullptr, "indices is NULL");
+  JPT_REQUIRE(g.total_pages > 0 && g.page_size > 0, "total_pages and page_size must be positive");
+  int32_t st = check_quant_common(g.heads, g.dim, g.in_dtype, g.scale_dtype, g.scale_heads, g.rounding);
+  if (st != JPT_OK) return st;
+  QuantParams p{};
+  p.a.new_k = g.new_k;
+  p.a.new_v = g.new_v;
+  p.a.cache_k = g.pages_k;
+  p.a.cache_v = g.pages_v;
+  p.a.k_scale = g.k_scale_pages;
+  p.a.v_scale = g.v_scale_pages;
+  p.a.batch = g.batch;
+  p.a.heads = g.heads;
+  p.a.dim = g.dim;
+  p.a.in_dtype = g.in_dtype;
+  p.a.scale_dtype = g.scale_dtype;
+  p.a.scale_heads = g.scale_heads;
+  p.a.rounding = g.rounding;
+  p.indices = g.indices;
+  p.n_active = g.n_active;
+  p.total_pages = g.total_pages;
+  p.page_size = g.page_size;
+  return launch_quant(p, g.n_active, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

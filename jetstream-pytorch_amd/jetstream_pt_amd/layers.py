@@ -1,0 +1,114 @@
+"""Decode-step attention orchestration: cache update, attention, new-token merge.
+
+AttentionKernel and Int8KVAttentionKernel keep the reference's constructor and
+call signature (jetstream_pt/layers.py:382-550, :553-718): cache.update(), then
+attention over the returned cache by the implementation the mode flags pick
+(ragged / flash / paged / dense), then - in lazy-update mode - the step's own
+token attended separately and merged by log-sum-exp.
+
+With `fuse_new_token` (default) the ragged path hands the new token to the
+attention launch itself, which merges it in its epilogue; the unfused sequence
+(second flash_attention call + lse_merge) stays available and is what the
+other lazy combinations use.  Only this attention part of the reference's
+layers.py is provided; projections, RoPE and norms are outside the KV path.
+"""
+
+import torch
+
+from . import attention_kernel as ak
+
+
+class AttentionKernel:
+
+  def __init__(self, env, layer_id, *, sm_scale_paged=1.0, fuse_new_token=True):
+    self.env = env
+    self.layer_id = layer_id
+    self.sm_scale_paged = sm_scale_paged
+    self.fuse_new_token = fuse_new_token
+    self.dense_attention = ak.dense_attention
+    self.flash_attention = ak.flash_attention
+    self.page_attention = ak.call_paged_attention
+    self.ragged_attention_orig = ak.RaggedAttentionKernel(env)
+    self.ragged_attention_new = ak.RaggedAttentionKernel(env)
+
+  def _attend(self, xq, keys, values, k_scaler, v_scaler, local_mask, cache, start, end,
+              ragged_batch_index, ragged_block_index, new_token=None):
+    env = self.env
+    bsz, num_heads, seqlen, head_dim = xq.shape
+    local_max = local_denom = None
+    if env.ragged_mha and seqlen == 1 and keys.shape[-2] > 1:
+      impl = self.ragged_attention_new if keys.dim() == 4 else self.ragged_attention_orig
+      local_output, (local_max, local_denom) = impl(
+          xq, keys, values, self.layer_id, start, end, ragged_batch_index, ragged_block_index,
+          k_scaler, v_scaler, **(new_token or {}))
+    elif env.flash_attention and seqlen == 1:
+      local_output, (local_max, local_denom) = self.flash_attention(
+          xq=xq, keys=keys, values=values, layer=self.layer_id, k_scaler=k_scaler,
+          v_scaler=v_scaler, mask=local_mask)
+    elif env.page_attention and seqlen == 1 and hasattr(cache, "page_attention_manager"):
+      pam = cache.page_attention_manager
+      lengths, page_indices = pam.device_tables(xq.device)
+      local_output = self.page_attention(
+          env, torch.squeeze(xq, 2), keys, values, lengths, page_indices,
+          sm_scale=self.sm_scale_paged, k_scaler=k_scaler, v_scaler=v_scaler)
+    else:
+      local_output = self.dense_attention(
+          xq=xq, keys=keys, values=values, k_scaler=k_scaler, v_scaler=v_scaler, mask=local_mask)
+    local_output = local_output.reshape(bsz, num_heads, seqlen, head_dim)
+    if local_max is not None:
+      local_max = local_max.reshape(bsz, num_heads, seqlen, 1)
+      local_denom = local_denom.reshape(bsz, num_heads, seqlen, 1)
+    return local_output, (local_max, local_denom)
+
+  def _will_fuse(self, seqlen, keys):
+    env = self.env
+    return (self.fuse_new_token and env.lazy_cache_update and seqlen == 1 and env.ragged_mha
+            and keys.shape[-2] > 1)
+
+  def __call__(self, xq, xk, xv, mask, cache, start=None, end=None, ragged_batch_index=None,
+               ragged_block_index=None):
+    """xq (batch, heads, seqlen, head_dim); xk, xv (batch, kv_heads, seqlen, head_dim);
+    mask additive 0/-inf or None; cache a CacheInterface object."""
+    seqlen = xq.shape[2]
+    orig_keys, orig_values = cache.update(xk, xv, self.layer_id)
+    args = (cache, start, end, ragged_batch_index, ragged_block_index)
+    if self._will_fuse(seqlen, orig_keys):
+      dt = orig_keys.dtype
+      new = dict(new_key=xk.to(dt).contiguous(), new_value=xv.to(dt).contiguous())
+      return self._attend(xq, orig_keys, orig_values, None, None, mask, *args, new_token=new)[0]
+    existing_output, (existing_max, existing_denom) = self._attend(
+        xq, orig_keys, orig_values, None, None, mask, *args)
+    if not self.env.lazy_cache_update or seqlen > 1:
+      return existing_output
+    new_output, (new_max, new_denom) = self._attend(xq, xk, xv, None, None, None, *args)
+    return ak.lse_merge(existing_output, existing_max, existing_denom, new_output, new_max,
+                        new_denom)
+
+
+class Int8KVAttentionKernel(AttentionKernel):
+
+  def __call__(self, xq, xk, xv, mask, cache, start=None, end=None, ragged_batch_index=None,
+               ragged_block_index=None):
+    seqlen = xq.shape[2]
+    ret = cache.update(xk, xv, self.layer_id)
+    if len(ret) == 4:  # int8 pages: (codes k, codes v, scale pages k, scale pages v)
+      orig_keys, orig_values, k_scaler, v_scaler = ret
+      new_key = new_value = new_k_scaler = new_v_scaler = None
+    else:
+      (orig_keys, orig_values, new_key, new_value, k_scaler, v_scaler, new_k_scaler,
+       new_v_scaler) = ret
+    args = (cache, start, end, ragged_batch_index, ragged_block_index)
+    if new_key is not None and self._will_fuse(seqlen, orig_keys):
+      new = dict(new_key=new_key, new_value=new_value, new_k_scaler=new_k_scaler,
+                 new_v_scaler=new_v_scaler)
+      return self._attend(xq, orig_keys, orig_values, k_scaler, v_scaler, mask, *args,
+                          new_token=new)[0]
+    existing_output, (existing_max, existing_denom) = self._attend(
+        xq, orig_keys, orig_values, k_scaler, v_scaler, mask, *args)
+    if not self.env.lazy_cache_update or seqlen > 1:
+      return existing_output
+    # over the QUANTISED new token, as the reference does (layers.py:704-706)
+    new_output, (new_max, new_denom) = self._attend(
+        xq, new_key, new_value, new_k_scaler, new_v_scaler, None, *args)
+    return ak.lse_merge(existing_output, existing_max, existing_denom, new_output, new_max,
+                        new_denom)

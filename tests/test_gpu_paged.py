@@ -1,0 +1,154 @@
+"""GPU parity: paged cache insert / append / gather through the C ABI against
+the reference's exact-integer scenarios and the CPU oracle (bit-exact)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import Env as OEnv
+from oracle import kv_cache as okv
+from oracle import quant as oquant
+from oracle.page_manager import PageAttentionManager as OraclePAM
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def genv(pages, ps):
+  from jetstream_pt_amd.environment import JetEngineEnvironment, JetEngineEnvironmentData
+  return JetEngineEnvironment(JetEngineEnvironmentData(
+      paged_attention_total_num_pages=pages, paged_attention_page_size=ps))
+
+
+def make(cfg):
+  from jetstream_pt_amd.page_attention_manager import PageAttentionManager
+  return PageAttentionManager(cfg["batch_size"], cfg["total_num_pages"], cfg["page_size"],
+                              cfg["max_pages_per_sequence"])
+
+
+def insert(pam, pages, seq_len, dim, slot):
+  from jetstream_pt_amd.cache_manager import KVCachePrefill
+  kv = torch.arange(seq_len * dim).reshape(1, 1, seq_len, dim).to(torch.bfloat16).to(DEV)
+  pre = KVCachePrefill()
+  pre.update(kv, kv, 0)
+  num_pages, idx = pam.reserve_pages_insert(slot, seq_len)
+  return pam.insert_prefill_cache([pre.state()], [pages], idx)
+
+
+@pytest.mark.parametrize("name", ["prefill_insert", "prefill_insert_multiple_pages"])
+def test_kat_prefill_insert(kats, name):
+  from jetstream_pt_amd.cache_manager import PageKVCacheGenerate
+  k = kats[name]
+  pam = make(k["manager"])
+  cache = PageKVCacheGenerate.empty(tuple(k["pages_shape"]), DEV, genv(20, 4))
+  (pk, pv), = insert(pam, cache.state(), k["seq_len"], 2, k["slot"])
+  for pages in (pk.cpu(), pv.cpu()):
+    if name == "prefill_insert":
+      assert pages[0, 0].tolist() == k["expected_page0"]
+    else:
+      assert pages[0, 0:2].tolist() == k["expected_pages_0_1"]
+      lo, hi = k["untouched_pages"]
+      assert torch.count_nonzero(pages[0, lo:hi]) == 0
+
+
+def test_kat_page_attention_update(kats):
+  from jetstream_pt_amd.cache_manager import PageKVCacheGenerate
+  k = kats["page_attention_update"]
+  pam = make(k["manager"])
+  env = genv(20, 4)
+  cache = PageKVCacheGenerate.empty(tuple(k["pages_shape"]), DEV, env)
+  pages = cache.state()
+  for seq_len, slot in k["prefill_inserts_seq_len_slot"]:
+    insert(pam, pages, seq_len, k["prefill_dim"], slot)
+  lens = np.asarray(k["lens"])
+  pam.fill_new_pages(lens)
+  pti = pam.get_page_token_indices(lens)
+  obj = PageKVCacheGenerate(pages[0], pages[1], pam, torch.from_numpy(pti).to(DEV), None, env=env)
+  new = torch.arange(-1, -11, -1).reshape(5, 1, 1, 2).to(torch.bfloat16).to(DEV)
+  rk, rv = obj.update(new, new)
+  for p in (rk.cpu(), rv.cpu()):
+    assert p[0, 0].tolist() == k["expected_page0"]
+    assert p[0, 7].tolist() == k["expected_page7"]
+    assert p[0, 6].tolist() == k["expected_page6"]
+
+
+@pytest.mark.parametrize("dtype,dim", [(torch.bfloat16, 128), (torch.float32, 6), (torch.bfloat16, 3)])
+def test_random_paged_lifecycle_matches_oracle(dtype, dim):
+  """Seeded free list, inserts, 20 decode steps of fill / indices / append,
+  then every slot gathered back: pages and gathers bit-exact."""
+  from jetstream_pt_amd.cache_manager import PageKVCacheGenerate
+  from jetstream_pt_amd.page_attention_manager import PageAttentionManager
+  g = torch.Generator().manual_seed(200)
+  rng = np.random.default_rng(200)
+  b, h, p, ps, mp = 8, 3, 64, 8, 6
+  order = rng.permutation(p).astype(np.int32)
+  gp = PageAttentionManager(b, p, ps, mp, free_list_order=order)
+  op = OraclePAM(b, p, ps, mp, free_list_order=order)
+  env = genv(p, ps)
+  oenv = OEnv(paged_attention_total_num_pages=p, paged_attention_page_size=ps)
+  base = torch.randn((h, p, ps, dim), generator=g).to(dtype)  # stale contents must survive where untouched
+  ok_, ov_ = base.clone(), (base * 2).clone()
+  gk_, gv_ = ok_.to(DEV), ov_.to(DEV)
+  lens = np.array([5, 0, 8, 17, 16, 1, 0, 24], dtype=np.int32)
+  for slot, n in enumerate(lens):
+    if n:
+      k = torch.randn((1, h, int(n), dim), generator=g).to(dtype)
+      v = torch.randn((1, h, int(n), dim), generator=g).to(dtype)
+      _, gi = gp.reserve_pages_insert(slot, int(n))
+      _, oi = op.reserve_pages_insert(slot, int(n))
+      assert gi.tolist() == oi.tolist()
+      gp.insert_prefill_cache([(k.to(DEV), v.to(DEV))], [(gk_, gv_)], gi)
+      op.insert_prefill_cache([(k, v)], [(ok_, ov_)], oi)
+  assert torch.equal(gk_.cpu(), ok_) and torch.equal(gv_.cpu(), ov_)
+  for _ in range(20):
+    gp.fill_new_pages(lens)
+    op.fill_new_pages(lens)
+    gi, oi = gp.get_page_token_indices(lens), op.get_page_token_indices(lens)
+    assert gi.tolist() == oi.tolist()
+    nk = torch.randn((b, h, 1, dim), generator=g).to(dtype)
+    nv = torch.randn((b, h, 1, dim), generator=g).to(dtype)
+    PageKVCacheGenerate(gk_, gv_, gp, gi, None, env=env).update(nk.to(DEV), nv.to(DEV))
+    okv.PageKVCacheGenerate(ok_, ov_, op, torch.from_numpy(oi), None, env=oenv).update(nk, nv)
+    lens = np.where(lens == 0, 0, lens + 1).astype(np.int32)
+  assert torch.equal(gk_.cpu(), ok_) and torch.equal(gv_.cpu(), ov_)
+  for slot in range(b):
+    (gk, gv), = gp.get_compress_kv_cache([(gk_, gv_)], slot)
+    (wk, wv), = op.get_compress_kv_cache([(ok_, ov_)], slot)
+    assert gk.shape == wk.shape and torch.equal(gk.cpu(), wk) and torch.equal(gv.cpu(), wv)
+
+
+@pytest.mark.parametrize("hs,sdt", [(1, torch.float32), (2, torch.bfloat16)])
+def test_int8_pages_equal_quantise_then_row_write(hs, sdt):
+  """int8 pages (no reference class): codes/scales must equal the decode
+  quantiser's output written by the paged row scatter."""
+  from jetstream_pt_amd.cache_manager import Int8PageKVCacheGenerate
+  from jetstream_pt_amd.page_attention_manager import PageAttentionManager
+  g = torch.Generator().manual_seed(201)
+  b, h, p, ps, d = 6, 2, 32, 32, 128
+  pam = PageAttentionManager(b, p, ps, 4)
+  lens = np.array([5, 0, 32, 33, 64, 1], dtype=np.int32)
+  for slot, n in enumerate(lens):
+    if n:
+      pam.reserve_pages_insert(slot, int(n))
+  pam.fill_new_pages(lens)
+  pti = pam.get_page_token_indices(lens)
+  cache = Int8PageKVCacheGenerate.empty((h, p, ps, d), DEV, genv(p, ps), scale_heads=hs, scale_dtype=sdt)
+  cache.page_attention_manager, cache.page_token_indices = pam, pti
+  nk = torch.randn((b, h, 1, d), generator=g).to(torch.bfloat16)
+  nv = torch.randn((b, h, 1, d), generator=g).to(torch.bfloat16)
+  ck, cv, ks, vs = cache.update(nk.to(DEV), nv.to(DEV))
+  cdt = None if sdt == torch.bfloat16 else sdt
+  wkq, wks = oquant.quantize_decode(nk, hs, cdt)
+  wvq, wvs = oquant.quantize_decode(nv, hs, cdt)
+  want_k = torch.zeros((h, p, ps, d), dtype=torch.int8)
+  want_v = torch.zeros((h, p, ps, d), dtype=torch.int8)
+  want_ks = torch.ones((hs, p, ps), dtype=sdt)
+  want_vs = torch.ones((hs, p, ps), dtype=sdt)
+  for j in range(pti.shape[1]):
+    page, tok, slot = (int(x) for x in pti[:, j])
+    want_k[:, page, tok % ps] = wkq[slot, :, 0]
+    want_v[:, page, tok % ps] = wvq[slot, :, 0]
+    want_ks[:, page, tok % ps] = wks[slot, :, 0, 0]
+    want_vs[:, page, tok % ps] = wvs[slot, :, 0, 0]
+  assert torch.equal(ck.cpu(), want_k) and torch.equal(cv.cpu(), want_v)
+  assert torch.equal(ks.cpu(), want_ks) and torch.equal(vs.cpu(), want_vs)
