@@ -155,6 +155,8 @@ class PageAttentionManager:
     heads, total, ps, dim = cache.shape
     row = _ffi.as_i32(indices, cache.device)
     out = torch.empty((heads, lens, dim), dtype=cache.dtype, device=cache.device)
+    if lens == 0:
+      return out
     _ffi.check(_ffi.lib.jpt_paged_gather(
         _ffi.ptr(out), _ffi.ptr(cache), _ffi.ptr(row), lens, heads, total, ps,
         dim * cache.element_size(), _ffi.stream()))
