@@ -11,7 +11,7 @@ import queue
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libjpt_mi355.so")
+LIB_PATH = os.environ.get("JPT_MI355_LIB") or os.path.join(_HERE, "libjpt_mi355.so")
 
 if not os.path.exists(LIB_PATH):
   raise ImportError(
