@@ -17,7 +17,8 @@ OUT_DIR = os.path.join(HERE, "jetstream_pt_amd")
 LIB = os.path.join(OUT_DIR, "libjpt_mi355.so")
 BUILD = os.path.join(HERE, "build")
 
-SOURCES = ["api.cpp", "pam.cpp", "kv_lines.hip", "paged_kv.hip", "attn_generic.hip", "attn_decode.hip"]
+SOURCES = ["api.cpp", "pam.cpp", "kv_lines.hip", "paged_kv.hip", "attn_generic.hip", "attn_decode.hip",
+           "attn_decode_i8.hip", "attn_decode_bf16.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -43,7 +44,7 @@ def _compile(src):
 
 def build(verbose=True):
   os.makedirs(BUILD, exist_ok=True)
-  with concurrent.futures.ThreadPoolExecutor(max_workers=min(6, os.cpu_count() or 1)) as ex:
+  with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as ex:
     objs = list(ex.map(_compile, SOURCES))
   tmp = LIB + ".tmp"
   cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]
