@@ -55,9 +55,13 @@ constexpr int kThreads = kWaves * 64;
 constexpr int kSideBytes = 512;     // ks | vs | mask, 128 bytes each at most
 constexpr int kOStride = 140;       // padded LDS row of 128 outputs
 constexpr int kLdsBudget = 80 * 1024 - 256;  // two workgroups per compute unit
-constexpr int kSpinLimit = 1 << 20;
+constexpr int kSpinLimit = 1 << 18;  // tens of milliseconds
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
+
+// 2^x by the hardware instruction alone.  Arguments here are <= 0 (or -inf);
+// results below the normal range flush to zero, which is right for them.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // column d = 32g + c of an output row lives at 33g + c, so the 16 writers of a
 // wave (4 rows x 4 column groups) hit distinct banks
@@ -220,11 +224,28 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   __shared__ int sm_folded[C::kFoldBufs];
   __shared__ int sm_abort;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  __shared__ int sm_simd[kWaves];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int hw_wave = tid >> 6;
   if (tid < C::kSlots) { sm_filled[tid] = 0; sm_freed[tid] = 0; }
   if (tid < C::kFoldBufs) { sm_arrived[tid] = 0; sm_folded[tid] = 0; }
   if (tid == 0) sm_abort = 0;
+  if (lane == 0) sm_simd[hw_wave] = (__builtin_amdgcn_s_getreg(0xF804) >> 4) & 3;  // HW_REG_HW_ID: SIMD_ID
   __syncthreads();
+  // Roles.  The producer is nearly idle, so the two workgroups sharing a
+  // compute unit should not both park theirs on the same SIMD: pick the wave
+  // that runs on a SIMD derived from the workgroup id (workgroups j and j+32
+  // of an XCD share a unit), if there is one.  `wave` is the role index:
+  // consumers 0..kConsumers-1, producer kConsumers.
+  int producer_wave;
+  {
+    const int j = blockIdx.x >> 3;
+    const int want = (((j >> 5) & 1) << 1) | (j & 1);
+    producer_wave = want % kWaves;
+    for (int w = kWaves - 1; w >= 0; --w)
+      if (sm_simd[w] == want) producer_wave = w;
+  }
+  const int wave = hw_wave == producer_wave ? kConsumers : hw_wave - (hw_wave > producer_wave ? 1 : 0);
 
   const int R = p.rows;
   const int G = gridDim.x;  // multiple of 8
@@ -475,11 +496,11 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
     const float m_new = fmaxf(m_run, tmax);
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = exp2f(m_run - m_use);
+    const float alpha = fast_exp2(m_run - m_use);
     float w[8], psum = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const float pr = exp2f(sc[i] - m_use);
+      const float pr = fast_exp2(sc[i] - m_use);
       psum += pr;
       w[i] = SCALE ? (live[i] ? pr * vs[i] : 0.f) : pr;
     }
