@@ -257,6 +257,12 @@ int32_t attn_fast_launch(const jpt_attn_args& a, AttnMode mode, hipStream_t stre
   p.rows = rows;
   p.rep = rep;
   p.total_items = l.max_entries * a.kv_heads;
+#ifdef JPT_ATTN_TRACE
+  {
+    const char* e = getenv("JPT_TRACE_PTR");
+    p.trace = e ? reinterpret_cast<unsigned long long*>(strtoull(e, nullptr, 0)) : nullptr;
+  }
+#endif
   if (!a.reuse_plan) {
     int32_t st = attn_plan_launch(a, mode == kPaged, stream);
     if (st != JPT_OK) return st;

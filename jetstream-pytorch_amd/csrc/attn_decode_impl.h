@@ -63,9 +63,9 @@ constexpr float kLn2 = 0.6931471805599453f;
 // results below the normal range flush to zero, which is right for them.
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// column d = 32g + c of an output row lives at 33g + c, so the 16 writers of a
-// wave (4 rows x 4 column groups) hit distinct banks
-__device__ __forceinline__ int o_col(int d) { return d + (d >> 5); }
+// column d = 32g + c of an output row lives at 36g + c: the column groups of a
+// wave's writers fall on different banks and runs of eight stay 16-byte aligned
+__device__ __forceinline__ int o_col(int d) { return d + 4 * (d >> 5); }
 
 enum ScaleKind { kNoScale = 0, kScaleF32 = 1, kScaleBF16 = 2 };
 
@@ -98,7 +98,7 @@ __device__ __forceinline__ int lds_peek(const int* p) {
 }
 __device__ __forceinline__ void lds_poke(int* p, int v) {
   const uint32_t addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_int_ptr)p));
-  asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : : "v"(addr), "v"(v) : "memory");
+  asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(v) : "memory");
 }
 
 // Load through the scalar data path.  `p` must be the same in every lane and
@@ -204,6 +204,14 @@ struct Tile<__bf16> {
   }
 };
 
+// Per-wave timing records for development builds (-DJPT_ATTN_TRACE): eight
+// 64-bit words per wave, times in ticks of the 100 MHz real-time counter.
+#ifdef JPT_ATTN_TRACE
+#define JPT_TR(stmt) stmt
+#else
+#define JPT_TR(stmt)
+#endif
+
 // One work item: a chunk of one slot for one KV head.
 struct Item {
   int slot, start, count, part, n_chunks, h;
@@ -215,7 +223,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   using C = Config<KV, SCALE, MASK, RC>;
   const jpt_attn_args& a = p.a;
   __shared__ __attribute__((aligned(1024))) char ring[C::kSlots * C::kSlotBytes];
-  __shared__ float sm_o[C::kFoldBufs][kConsumers][RC][kOStride];
+  __shared__ __attribute__((aligned(16))) float sm_o[C::kFoldBufs][kConsumers][RC][kOStride];
   __shared__ float sm_m[C::kFoldBufs][kConsumers][RC];
   __shared__ float sm_l[C::kFoldBufs][kConsumers][RC];
   __shared__ int sm_filled[C::kSlots];   // times the producer filled this slot
@@ -227,6 +235,8 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   __shared__ int sm_simd[kWaves];
   const int tid = threadIdx.x, lane = tid & 63;
   const int hw_wave = tid >> 6;
+  JPT_TR(const unsigned long long tr_start = __builtin_amdgcn_s_memrealtime();)
+  JPT_TR(unsigned long long tr_wait = 0; unsigned long long tr_fold = 0; unsigned long long tr_first = 0; unsigned long long tr_t = 0; int tr_tiles = 0;)
   if (tid < C::kSlots) { sm_filled[tid] = 0; sm_freed[tid] = 0; }
   if (tid < C::kFoldBufs) { sm_arrived[tid] = 0; sm_folded[tid] = 0; }
   if (tid == 0) sm_abort = 0;
@@ -298,7 +308,30 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     constexpr int kPieces = C::kRowBytes / 16;       // 16-byte pieces per row
     constexpr int kRowsPerLoad = 64 / kPieces;       // rows one load instruction covers
     constexpr int kLoadsPerMatrix = C::kTileBytes / 1024;
+    // Lane l of load j fills LDS piece slot 64j + l: row t = 64j / kPieces +
+    // l / kPieces, piece slot l % kPieces, with the global piece chosen by the
+    // bank swizzle.  Rows past the chunk end repeat its last row (keeps every
+    // access inside the cache and its contents finite).
+    int row_of[kLoadsPerMatrix];
+    uint32_t piece_off[kLoadsPerMatrix];
+#pragma unroll
+    for (int j = 0; j < kLoadsPerMatrix; ++j) {
+      row_of[j] = j * kRowsPerLoad + lane / kPieces;
+      piece_off[j] = static_cast<uint32_t>(((lane % kPieces) ^ (row_of[j] & (kPieces - 1))) * 16);
+    }
+    // scales, one load for both rows: float32 - lanes 0..31 k, 32..63 v;
+    // bf16 - lanes 0..15 k, 16..31 v (two positions per lane)
+    constexpr int kHalf = SCALE == kScaleF32 ? 32 : 16;
+    const char* scale_lane = nullptr;
+    if (SCALE) {
+      const bool is_v = lane >= kHalf;
+      scale_lane = static_cast<const char*>(is_v ? a.v_scale : a.k_scale) + (lane - (is_v ? kHalf : 0)) * 4;
+    }
+    constexpr int kEs = SCALE == kScaleF32 ? 4 : 2;
+
     int issued = 0, signalled = 0;
+    int fill_slot = 0, fill_round = 0;    // issued % kSlots, issued / kSlots
+    int sig_slot = 0, sig_round = 1;      // signalled % kSlots, signalled / kSlots + 1
     // Hands every tile that has landed to the consumers.  Loads complete in
     // order, so with `out` loads still counted as outstanding (the wave's own
     // vector-memory counter, read without waiting) all tiles but the newest
@@ -308,8 +341,9 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       const int out = static_cast<int>((ib & 0xF) | (((ib >> 22) & 0x3) << 4));
       const int landed = issued - (out + C::kLoadsPerTile - 1) / C::kLoadsPerTile;
       while (signalled < landed) {
-        if (lane == 0) lds_poke(&sm_filled[signalled % C::kSlots], signalled / C::kSlots + 1);
+        if (lane == 0) lds_poke(&sm_filled[sig_slot], sig_round);
         ++signalled;
+        if (++sig_slot == C::kSlots) { sig_slot = 0; ++sig_round; }
       }
     };
     Item cur = fetch(0);
@@ -318,13 +352,46 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       const Item nxt2 = fetch(k + 2);  // entries are read two items ahead of their use
       const int hs = a.scale_heads == 1 ? 0 : cur.h;
       const int n_cache = cache_tiles(cur), nt = item_tiles(cur);
+      // rows of the item's first position in the key/value and scale tensors
+      const char *kt = nullptr, *vt = nullptr;
+      int64_t srow = 0;
+      int page = 0;
+      if (PAGED) {
+        page = load_uniform(a.page_table + (static_cast<int64_t>(cur.slot) * a.max_pages + cur.start / a.page_size));
+      } else {
+        const int64_t row0 = (static_cast<int64_t>(cur.slot) * a.kv_heads + cur.h) * a.seq + cur.start;
+        kt = static_cast<const char*>(a.k) + row0 * C::kRowBytes;
+        vt = static_cast<const char*>(a.v) + row0 * C::kRowBytes;
+        srow = (static_cast<int64_t>(cur.slot) * a.scale_heads + hs) * a.seq + cur.start;
+      }
       for (int ti = 0; ti < nt; ++ti) {
-        const int s = issued % C::kSlots;
+        const bool is_new = ti >= n_cache;
+        int valid = 1;  // the new token: every row of the tile is that one token
+        if (is_new) {
+          const int64_t row = static_cast<int64_t>(cur.slot) * a.kv_heads + cur.h;
+          kt = static_cast<const char*>(a.new_k) + row * C::kRowBytes;
+          vt = static_cast<const char*>(a.new_v) + row * C::kRowBytes;
+          srow = 0;  // its scales are read by the consumers; load the tensors' heads
+        } else {
+          const int t0 = cur.start + ti * kTile;
+          valid = min(kTile, cur.start + cur.count - t0);
+          if (PAGED) {  // a tile never straddles a page
+            const int64_t in_pool = static_cast<int64_t>(page) * a.page_size + t0 % a.page_size;
+            const int64_t row0 = static_cast<int64_t>(cur.h) * a.total_pages * a.page_size + in_pool;
+            kt = static_cast<const char*>(a.k) + row0 * C::kRowBytes;
+            vt = static_cast<const char*>(a.v) + row0 * C::kRowBytes;
+            srow = static_cast<int64_t>(hs) * a.total_pages * a.page_size + in_pool;
+            // page of the next tile, read while this one is issued
+            const int tn = min(t0 + kTile, cur.start + cur.count - 1);
+            page = load_uniform(a.page_table + (static_cast<int64_t>(cur.slot) * a.max_pages + tn / a.page_size));
+          }
+        }
         // wait for the slot's previous tile to be taken, handing over landed
         // tiles meanwhile
+        JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
         for (int spins = 0;; ++spins) {
           signal_landed();
-          if (lds_peek(&sm_freed[s]) >= issued / C::kSlots) break;
+          if (lds_peek(&sm_freed[fill_slot]) >= fill_round) break;
           if (spins > kSpinLimit || lds_peek(&sm_abort)) {
             lds_poke(&sm_abort, 1);
             __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
@@ -332,66 +399,31 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
           }
           __builtin_amdgcn_s_sleep(1);
         }
-        char* slot = ring + s * C::kSlotBytes;
-        const bool is_new = ti >= n_cache;
-        // rows of position t0 in the key/value and scale tensors
-        const char *kt, *vt;
-        int64_t srow0 = 0;
-        int valid;
-        const int t0 = cur.start + ti * kTile;
-        if (is_new) {
-          const int64_t row = static_cast<int64_t>(cur.slot) * a.kv_heads + cur.h;
-          kt = static_cast<const char*>(a.new_k) + row * C::kRowBytes;
-          vt = static_cast<const char*>(a.new_v) + row * C::kRowBytes;
-          valid = 1;  // every row of the tile is that one token, position 0 counts
-        } else {
-          int64_t row0;
-          if (PAGED) {  // a tile never straddles a page
-            const int page = load_uniform(a.page_table + (static_cast<int64_t>(cur.slot) * a.max_pages + t0 / a.page_size));
-            const int64_t in_pool = static_cast<int64_t>(page) * a.page_size + t0 % a.page_size;
-            row0 = static_cast<int64_t>(cur.h) * a.total_pages * a.page_size + in_pool;
-            srow0 = static_cast<int64_t>(hs) * a.total_pages * a.page_size + in_pool;
-          } else {
-            row0 = (static_cast<int64_t>(cur.slot) * a.kv_heads + cur.h) * a.seq + t0;
-            srow0 = (static_cast<int64_t>(cur.slot) * a.scale_heads + hs) * a.seq + t0;
-          }
-          kt = static_cast<const char*>(a.k) + row0 * C::kRowBytes;
-          vt = static_cast<const char*>(a.v) + row0 * C::kRowBytes;
-          valid = min(kTile, cur.start + cur.count - t0);
-        }
-        // K and V rows: lane l of load j fills LDS piece slot 64j + l, i.e. row
-        // t = (64j + l) / kPieces, piece slot l % kPieces, with the global piece
-        // chosen by the bank swizzle.  Rows past the chunk end repeat its last
-        // row (keeps every access inside the cache and its contents finite).
+        JPT_TR(tr_wait += __builtin_amdgcn_s_memrealtime() - tr_t; if (!tr_first) tr_first = __builtin_amdgcn_s_memrealtime() - tr_start;)
+        char* slot = ring + fill_slot * C::kSlotBytes;
 #pragma unroll
         for (int j = 0; j < kLoadsPerMatrix; ++j) {
-          const int t = j * kRowsPerLoad + lane / kPieces;
-          const int piece = (lane % kPieces) ^ (t & (kPieces - 1));
-          const int64_t off = (is_new ? 0 : static_cast<int64_t>(min(t, valid - 1)) * C::kRowBytes) + piece * 16;
+          const uint32_t off = static_cast<uint32_t>(min(row_of[j], valid - 1)) * C::kRowBytes + piece_off[j];
           __builtin_amdgcn_global_load_lds((global_ptr)(kt + off), (lds_ptr)(slot + j * 1024), 16, 0, 0);
           __builtin_amdgcn_global_load_lds((global_ptr)(vt + off), (lds_ptr)(slot + C::kTileBytes + j * 1024), 16, 0, 0);
         }
         char* side = slot + 2 * C::kTileBytes;
         if (SCALE) {
-          // one load for both scale rows: float32 - lanes 0..31 k, 32..63 v;
-          // bf16 - lanes 0..15 k, 16..31 v (two positions per lane).  The new
-          // token's scales are read by the consumers; its tile loads the head
-          // of the scale tensors only to keep the load count per tile fixed.
-          constexpr int kHalf = SCALE == kScaleF32 ? 32 : 16;
-          constexpr int kEs = SCALE == kScaleF32 ? 4 : 2;
-          const bool is_v = lane >= kHalf;
-          const int e = lane - (is_v ? kHalf : 0);
-          const char* base = static_cast<const char*>(is_v ? a.v_scale : a.k_scale);
-          const int64_t first = is_new ? 0 : srow0;
           if (lane < 2 * kHalf)
-            __builtin_amdgcn_global_load_lds((global_ptr)(base + (first + e * (4 / kEs)) * kEs), (lds_ptr)side, 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((global_ptr)(scale_lane + srow * kEs), (lds_ptr)side, 4, 0, 0);
         }
         if (MASK) {
-          const float* src = static_cast<const float*>(a.mask) + cur.slot * a.mask_stride_b + (is_new ? 0 : t0);
+          const float* src = static_cast<const float*>(a.mask) + cur.slot * a.mask_stride_b + (is_new ? 0 : cur.start + ti * kTile);
           if (lane < kTile)
             __builtin_amdgcn_global_load_lds((global_ptr)(src + lane), (lds_ptr)(side + 256), 4, 0, 0);
         }
         ++issued;
+        if (++fill_slot == C::kSlots) { fill_slot = 0; ++fill_round; }
+        if (!PAGED) {
+          kt += kTile * C::kRowBytes;
+          vt += kTile * C::kRowBytes;
+          srow += kTile;
+        }
       }
       cur = nxt;
       nxt = nxt2;
@@ -405,6 +437,11 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       }
       __builtin_amdgcn_s_sleep(1);
     }
+    JPT_TR(if (p.trace && lane == 0) {
+      unsigned long long* o = p.trace + (static_cast<size_t>(blockIdx.x) * kWaves + wave) * 8;
+      o[0] = issued; o[1] = tr_wait; o[2] = 0; o[3] = __builtin_amdgcn_s_memrealtime() - tr_start;
+      o[4] = tr_start; o[5] = 0; o[6] = tr_first; o[7] = sm_simd[hw_wave];
+    })
     return;
   }
 
@@ -437,7 +474,9 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   int cur_slot = 0, cur_h = 0;  // of the item being consumed
   auto consume_tile = [&](int t, int valid, bool is_new) -> bool {
     const int s = t % C::kSlots;
+    JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
     if (!wait_for(&sm_filled[s], t / C::kSlots + 1)) return false;
+    JPT_TR(tr_wait += __builtin_amdgcn_s_memrealtime() - tr_t; ++tr_tiles; if (!tr_first) tr_first = __builtin_amdgcn_s_memrealtime() - tr_start;)
     const char* slot = ring + s * C::kSlotBytes;
     const char* side = slot + 2 * C::kTileBytes;
     Tile<KV> tile;
@@ -531,7 +570,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
 #pragma unroll
       for (int j = 0; j < 8; ++j)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) sm_o[buf][wave][r][33 * g + 8 * i + j] = acc[j][i];
+        for (int i = 0; i < 4; ++i) sm_o[buf][wave][r][o_col(32 * g + 8 * i + j)] = acc[j][i];
       if (g == 0) {
         sm_m[buf][wave][r] = m_run;
         sm_l[buf][wave][r] = l_row;
@@ -545,28 +584,38 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     const int64_t q_row0 = (static_cast<int64_t>(it.slot) * a.q_heads + it.h * p.rep) * a.q_rows;
     float* part = p.partials + (static_cast<int64_t>(it.part) * a.kv_heads + it.h) * R * kPartFloats;
-    for (int idx = lane; idx < R * kD; idx += 64) {
-      const int row = idx / kD, d = idx % kD;
+    // four rows a pass: 16 lanes a row, eight consecutive outputs a lane
+    const int d0 = 8 * (lane & 15);
+    for (int row = lane >> 4; row < R; row += 4) {
       float M = -INFINITY;
 #pragma unroll
       for (int w2 = 0; w2 < kConsumers; ++w2) M = fmaxf(M, sm_m[buf][w2][row]);
-      float o = 0.f, l = 0.f;
+      float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      float l = 0.f;
 #pragma unroll
       for (int w2 = 0; w2 < kConsumers; ++w2) {
         const float mw = sm_m[buf][w2][row];
-        const float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
-        o += sm_o[buf][w2][row][o_col(d)] * f;
+        const float f = mw == -INFINITY ? 0.f : fast_exp2(mw - M);
         l += sm_l[buf][w2][row] * f;
+        const float4* src = reinterpret_cast<const float4*>(&sm_o[buf][w2][row][o_col(d0)]);
+        const float4 x = src[0], y = src[1];
+        o[0] += x.x * f; o[1] += x.y * f; o[2] += x.z * f; o[3] += x.w * f;
+        o[4] += y.x * f; o[5] += y.y * f; o[6] += y.z * f; o[7] += y.w * f;
       }
       if (it.n_chunks == 1) {
-        static_cast<uint16_t*>(a.out)[(q_row0 + row) * kD + d] = f32_to_bf16_bits(l > 0.f ? o / l : 0.f);
-        if (d == 0) {
+        const float inv = l > 0.f ? 1.f / l : 0.f;
+        const uint4 packed = make_uint4(pack_bf16(o[0] * inv, o[1] * inv), pack_bf16(o[2] * inv, o[3] * inv),
+                                        pack_bf16(o[4] * inv, o[5] * inv), pack_bf16(o[6] * inv, o[7] * inv));
+        *reinterpret_cast<uint4*>(static_cast<uint16_t*>(a.out) + (q_row0 + row) * kD + d0) = packed;
+        if (d0 == 0) {
           if (a.out_max) a.out_max[q_row0 + row] = M * kLn2;
           if (a.out_denom) a.out_denom[q_row0 + row] = l;
         }
       } else {
-        part[row * kPartFloats + d] = o;
-        if (d == 0) {
+        float4* dst = reinterpret_cast<float4*>(part + row * kPartFloats + d0);
+        dst[0] = make_float4(o[0], o[1], o[2], o[3]);
+        dst[1] = make_float4(o[4], o[5], o[6], o[7]);
+        if (d0 == 0) {
           part[row * kPartFloats + kD] = M;
           part[row * kPartFloats + kD + 1] = l;
         }
@@ -599,8 +648,17 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       const int valid = is_new ? 1 : min(kTile, cur.count - ti * kTile);
       if (!consume_tile(base + ti, valid, is_new)) return;
     }
+    JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
     if (!finish_item(cur, k)) return;
-    if (!nxt.valid) break;
+    JPT_TR(tr_fold += __builtin_amdgcn_s_memrealtime() - tr_t;)
+    if (!nxt.valid) {
+      JPT_TR(if (p.trace && lane == 0) {
+        unsigned long long* o = p.trace + (static_cast<size_t>(blockIdx.x) * kWaves + wave) * 8;
+        o[0] = tr_tiles; o[1] = tr_wait; o[2] = tr_fold; o[3] = __builtin_amdgcn_s_memrealtime() - tr_start;
+        o[4] = tr_start; o[5] = k + 1; o[6] = tr_first; o[7] = sm_simd[hw_wave];
+      })
+      break;
+    }
     base += nt;
     cur = nxt;
     nxt = nxt2;

@@ -9,7 +9,7 @@ namespace jpt {
 constexpr int kTile = 32;        // positions per tile
 constexpr int kD = 128;          // head_dim
 constexpr int kMaxRows = 16;     // rep * q_rows
-constexpr int kPartFloats = kD + 2;  // a partial's row: o[128], max, sum
+constexpr int kPartFloats = kD + 4;  // a partial's row: o[128], max, sum, 2 unused (16-byte rows)
 
 struct PlanEntry {
   int32_t slot;        // -1: unused record
@@ -31,6 +31,9 @@ struct FastParams {
   int32_t rows;         // rep * q_rows
   int32_t rep;
   int32_t total_items;  // max_entries * kv_heads
+#ifdef JPT_ATTN_TRACE
+  unsigned long long* trace;  // per-wave timing records (development builds only)
+#endif
 };
 
 namespace decode {
