@@ -1,13 +1,15 @@
 // Streaming GQA decode attention kernel for gfx950, head_dim 128 (template
 // body; attn_decode_i8.hip and attn_decode_bf16.hip instantiate it).
 //
-// A persistent workgroup of four wavefronts walks its share of the planned
-// (chunk, KV head) items as one stream of 32-position tiles:
+// One workgroup per compute unit holds kGroups independent groups of
+// wavefronts; a group walks its share of the planned (chunk, KV head) items as
+// one stream of 32-position tiles:
 //
 //   producer wave   copies each tile's K rows, V rows and per-position scales
-//                   from HBM straight into an LDS ring with direct-to-LDS
-//                   loads (no registers), several tiles ahead and regardless
-//                   of item boundaries.  HBM sees full 1 KiB bursts of
+//                   from HBM straight into the group's LDS ring with
+//                   direct-to-LDS loads (no registers), several tiles ahead
+//                   and regardless of item boundaries, and each item's query
+//                   rows ahead of its first tile.  HBM sees full 1 KiB bursts of
 //                   contiguous cache rows; a first touch of a new cache row
 //                   (several microseconds with its TLB miss) is hidden behind
 //                   the tiles already in the ring.
@@ -21,15 +23,20 @@
 //                   probabilities that lane feeds to the second MFMA, so
 //                   probabilities never cross lanes.
 //
-// Waves never meet at a workgroup barrier: ring slots are handed over through
-// LDS counters, and the consumer that delivers the last part of an item folds
-// the three parts and writes the slot's output (one chunk) or parks the
+// A consumer wave is bound by latencies, not by issue slots, so the kernel
+// wants many of them per SIMD; several groups in one workgroup (instead of
+// several workgroups per unit) make the wave placement over the SIMDs even.
+// Waves never meet at a workgroup barrier after set-up: ring slots are handed
+// over through LDS counters, and the consumer that delivers the last part of an
+// item folds the parts and writes the slot's output (one chunk) or parks the
 // chunk's float32 partial (several; a second kernel folds those).  Every wait
 // is bounded: a wave that waits too long raises an abort flag and every wave
 // leaves, so a logic error shows up as wrong output, never as a hung GPU.
 #pragma once
 
 #include <math.h>
+
+#include <type_traits>
 
 #include "attn_common.h"
 #include "attn_plan.h"
@@ -39,6 +46,8 @@ namespace decode {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef const __attribute__((address_space(1))) void* global_ptr;
 typedef __attribute__((address_space(3))) void* lds_ptr;
@@ -46,15 +55,20 @@ typedef __attribute__((address_space(3))) void* lds_ptr;
 #ifndef JPT_ATTN_CONSUMERS
 #define JPT_ATTN_CONSUMERS 3
 #endif
+#ifndef JPT_ATTN_GROUPS
+#define JPT_ATTN_GROUPS 2
+#endif
 #ifndef JPT_ATTN_WAVES_PER_SIMD
 #define JPT_ATTN_WAVES_PER_SIMD 2
 #endif
 constexpr int kConsumers = JPT_ATTN_CONSUMERS;
-constexpr int kWaves = kConsumers + 1;
+constexpr int kGroups = JPT_ATTN_GROUPS;
+constexpr int kGroupWaves = kConsumers + 1;  // wave 0 of a group is its producer
+constexpr int kWaves = kGroups * kGroupWaves;
 constexpr int kThreads = kWaves * 64;
 constexpr int kSideBytes = 512;     // ks | vs | mask, 128 bytes each at most
 constexpr int kOStride = 140;       // padded LDS row of 128 outputs
-constexpr int kLdsBudget = 80 * 1024 - 256;  // two workgroups per compute unit
+constexpr int kLdsBudget = 160 * 1024 / kGroups - 512;  // per group; one workgroup per compute unit
 constexpr int kSpinLimit = 1 << 18;  // tens of milliseconds
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -76,11 +90,18 @@ struct Config {
   static constexpr int kTileBytes = kTile * kRowBytes;            // K or V of one tile
   static constexpr int kSlotBytes = 2 * kTileBytes + kSideBytes;
   static constexpr int kLoadsPerTile = 2 * kTileBytes / 1024 + (SCALE ? 1 : 0) + (MASK ? 1 : 0);
-  static constexpr int kFoldBufs = ((RC > 8 && kElem > 1) || kConsumers > 3) ? 1 : 2;
-  static constexpr int kFoldBytes = kFoldBufs * kConsumers * RC * (kOStride + 2) * 4;
-  static constexpr int kSlotsByLds = (kLdsBudget - kFoldBytes) / kSlotBytes;
-  static constexpr int kSlotsByCount = 63 / kLoadsPerTile;  // the load counter counts to 63
-  // ring slots: every one may hold a tile in flight
+  // query rows of the next items, staged by the producer
+  static constexpr int kQBufs = RC <= 8 ? 4 : 2;
+  static constexpr int kQBytes = kQBufs * RC * kD * 2;
+  static constexpr int kQLoadsMax = (RC + 3) / 4;  // 1 KiB (four rows) a load
+  static constexpr int kFoldPart = kConsumers * RC * (kOStride + 2) * 4;
+  // ring slots: every one may hold a tile in flight, and the wave's load
+  // counter counts to 63
+  static constexpr int kSlotsByCount = (63 - kQLoadsMax) / kLoadsPerTile;
+  static constexpr int kSlotsWith2 = (kLdsBudget - kQBytes - 2 * kFoldPart) / kSlotBytes;
+  static constexpr int kEnough = kSlotsByCount < 5 ? kSlotsByCount : 5;
+  static constexpr int kFoldBufs = kSlotsWith2 >= kEnough ? 2 : 1;
+  static constexpr int kSlotsByLds = (kLdsBudget - kQBytes - kFoldBufs * kFoldPart) / kSlotBytes;
   static constexpr int kSlots = kSlotsByLds < kSlotsByCount ? kSlotsByLds : kSlotsByCount;
   static_assert(kSlots >= 2, "LDS ring too small");
 };
@@ -118,12 +139,14 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   bf16x2 t = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
   return __builtin_bit_cast(uint32_t, t);
 }
-__device__ __forceinline__ float sbyte(uint32_t w, int k) {
-  return static_cast<float>(static_cast<signed char>(w >> (8 * k)));
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+  f16x2 t = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
+  return __builtin_bit_cast(uint32_t, t);
 }
-__device__ __forceinline__ bf16x8 as_op(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+template <typename Op>
+__device__ __forceinline__ Op as_op(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
   uint4 u = make_uint4(a, b, c, d);
-  return __builtin_bit_cast(bf16x8, u);
+  return __builtin_bit_cast(Op, u);
 }
 
 // One tile in a consumer's registers.  Lane (r, g) holds elements [32g, 32g+32)
@@ -134,8 +157,18 @@ __device__ __forceinline__ bf16x8 as_op(uint32_t a, uint32_t b, uint32_t c, uint
 template <typename KV>
 struct Tile;
 
+// int8 codes enter the matrix cores as float16 without a conversion
+// instruction: with the sign bit flipped a code byte is u = code + 128, and
+// the halfword 0x6400 | u is the float16 number 1024 + u = code + 1152
+// exactly.  A byte permute builds two such halfwords at once.  The constant
+// 1152 is taken out again where it is a rank-one term: 1152 * sum(q) is the
+// same for every position of a query row (the score accumulators start from
+// its negative), and 1152 * sum(weights) per row is accumulated by one more
+// MFMA against a tile of ones and subtracted when the item is finished.
 template <>
 struct Tile<int8_t> {
+  typedef f16x8 Op;
+  static constexpr float kBias = 1152.f;
   uint4 ka[2], kb[2];
   uint2 v[8];
   __device__ __forceinline__ void read(const char* ks, const char* vs, int r, int g, const int* pos) {
@@ -143,7 +176,9 @@ struct Tile<int8_t> {
     for (int half = 0; half < 2; ++half) {
       const int t = r + 16 * half;
       const uint4* row = reinterpret_cast<const uint4*>(ks + t * 128);
-      const uint4 x = row[(2 * g) ^ (t & 7)], y = row[(2 * g + 1) ^ (t & 7)];
+      uint4 x = row[(2 * g) ^ (t & 7)], y = row[(2 * g + 1) ^ (t & 7)];
+      x.x ^= 0x80808080u; x.y ^= 0x80808080u; x.z ^= 0x80808080u; x.w ^= 0x80808080u;
+      y.x ^= 0x80808080u; y.y ^= 0x80808080u; y.z ^= 0x80808080u; y.w ^= 0x80808080u;
       if (half == 0) { ka[0] = x; ka[1] = y; } else { kb[0] = x; kb[1] = y; }
     }
 #pragma unroll
@@ -152,23 +187,37 @@ struct Tile<int8_t> {
       v[i] = *reinterpret_cast<const uint2*>(vs + t * 128 + 16 * ((r >> 1) ^ (t & 7)) + 8 * (r & 1));
     }
   }
-  __device__ __forceinline__ bf16x8 k_op(bool second, int kk) const {
+  // bytes (b0, b1) or (b2, b3) of w as two float16 1024 + b
+  __device__ __forceinline__ static uint32_t widen(uint32_t w, bool upper) {
+    return __builtin_amdgcn_perm(0x64646464u, w, upper ? 0x04030402u : 0x04010400u);
+  }
+  __device__ __forceinline__ Op k_op(bool second, int kk) const {
     const uint4& q = second ? kb[kk >> 1] : ka[kk >> 1];
     const uint32_t w0 = (kk & 1) ? q.z : q.x, w1 = (kk & 1) ? q.w : q.y;
-    return as_op(pack_bf16(sbyte(w0, 0), sbyte(w0, 1)), pack_bf16(sbyte(w0, 2), sbyte(w0, 3)),
-                 pack_bf16(sbyte(w1, 0), sbyte(w1, 1)), pack_bf16(sbyte(w1, 2), sbyte(w1, 3)));
+    return as_op<Op>(widen(w0, false), widen(w0, true), widen(w1, false), widen(w1, true));
   }
-  __device__ __forceinline__ float v_elem(int i, int j) const {
-    return sbyte(j < 4 ? v[i].x : v[i].y, j & 3);
+  // byte j of positions 2i and 2i+1, sign bits flipped and the exponent set in one xor
+  __device__ __forceinline__ uint32_t v_pair(int i, int j) const {
+    const uint32_t lo = j < 4 ? v[2 * i].x : v[2 * i].y, hi = j < 4 ? v[2 * i + 1].x : v[2 * i + 1].y;
+    const uint32_t sel = 0x0c000c00u | static_cast<uint32_t>(j & 3) | (static_cast<uint32_t>(4 + (j & 3)) << 16);
+    return __builtin_amdgcn_perm(hi, lo, sel) ^ 0x64806480u;
   }
-  __device__ __forceinline__ bf16x8 v_op(int j) const {
-    return as_op(pack_bf16(v_elem(0, j), v_elem(1, j)), pack_bf16(v_elem(2, j), v_elem(3, j)),
-                 pack_bf16(v_elem(4, j), v_elem(5, j)), pack_bf16(v_elem(6, j), v_elem(7, j)));
+  __device__ __forceinline__ Op v_op(int j) const {
+    return as_op<Op>(v_pair(0, j), v_pair(1, j), v_pair(2, j), v_pair(3, j));
+  }
+  __device__ __forceinline__ static f32x4 mfma(Op a, Op b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  __device__ __forceinline__ static uint32_t pack(float lo, float hi) { return pack_f16(lo, hi); }
+  __device__ __forceinline__ static Op ones() {
+    return as_op<Op>(0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u);
   }
 };
 
 template <>
 struct Tile<__bf16> {
+  typedef bf16x8 Op;
+  static constexpr float kBias = 0.f;
   uint4 ka[4], kb[4];
   uint4 v[8];
   __device__ __forceinline__ void read(const char* ks, const char* vs, int r, int g, const int* pos) {
@@ -188,20 +237,25 @@ struct Tile<__bf16> {
       v[i] = *reinterpret_cast<const uint4*>(vs + t * 256 + 16 * (r ^ (t & 15)));
     }
   }
-  __device__ __forceinline__ bf16x8 k_op(bool second, int kk) const {
-    return __builtin_bit_cast(bf16x8, second ? kb[kk] : ka[kk]);
+  __device__ __forceinline__ Op k_op(bool second, int kk) const {
+    return __builtin_bit_cast(Op, second ? kb[kk] : ka[kk]);
   }
   __device__ __forceinline__ uint32_t v_word(int i, int j) const {
     const int w = j >> 1;
     return w == 0 ? v[i].x : w == 1 ? v[i].y : w == 2 ? v[i].z : v[i].w;
   }
-  __device__ __forceinline__ bf16x8 v_op(int j) const {
+  __device__ __forceinline__ Op v_op(int j) const {
     const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-    return as_op(__builtin_amdgcn_perm(v_word(1, j), v_word(0, j), sel),
-                 __builtin_amdgcn_perm(v_word(3, j), v_word(2, j), sel),
-                 __builtin_amdgcn_perm(v_word(5, j), v_word(4, j), sel),
-                 __builtin_amdgcn_perm(v_word(7, j), v_word(6, j), sel));
+    return as_op<Op>(__builtin_amdgcn_perm(v_word(1, j), v_word(0, j), sel),
+                     __builtin_amdgcn_perm(v_word(3, j), v_word(2, j), sel),
+                     __builtin_amdgcn_perm(v_word(5, j), v_word(4, j), sel),
+                     __builtin_amdgcn_perm(v_word(7, j), v_word(6, j), sel));
   }
+  __device__ __forceinline__ static f32x4 mfma(Op a, Op b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  __device__ __forceinline__ static uint32_t pack(float lo, float hi) { return pack_bf16(lo, hi); }
+  __device__ __forceinline__ static Op ones() { return as_op<Op>(0, 0, 0, 0); }  // unused
 };
 
 // Per-wave timing records for development builds (-DJPT_ATTN_TRACE): eight
@@ -222,54 +276,63 @@ template <typename KV, bool PAGED, int SCALE, bool MASK, int RC>
 __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode_kernel(FastParams p) {
   using C = Config<KV, SCALE, MASK, RC>;
   const jpt_attn_args& a = p.a;
-  __shared__ __attribute__((aligned(1024))) char ring[C::kSlots * C::kSlotBytes];
-  __shared__ __attribute__((aligned(16))) float sm_o[C::kFoldBufs][kConsumers][RC][kOStride];
-  __shared__ float sm_m[C::kFoldBufs][kConsumers][RC];
-  __shared__ float sm_l[C::kFoldBufs][kConsumers][RC];
-  __shared__ int sm_filled[C::kSlots];   // times the producer filled this slot
-  __shared__ int sm_freed[C::kSlots];    // times a consumer emptied it
-  __shared__ int sm_arrived[C::kFoldBufs];
-  __shared__ int sm_folded[C::kFoldBufs];
+  __shared__ __attribute__((aligned(1024))) char ring_all[kGroups][C::kSlots * C::kSlotBytes];
+  __shared__ __attribute__((aligned(16))) float sm_o_all[kGroups][C::kFoldBufs][kConsumers][RC][kOStride];
+  __shared__ __attribute__((aligned(16))) uint16_t sm_q_all[kGroups][C::kQBufs][RC][kD];
+  __shared__ float sm_m_all[kGroups][C::kFoldBufs][kConsumers][RC];
+  __shared__ float sm_l_all[kGroups][C::kFoldBufs][kConsumers][RC];
+  __shared__ int sm_filled_all[kGroups][C::kSlots];   // times the producer filled this slot
+  __shared__ int sm_freed_all[kGroups][C::kSlots];    // times a consumer emptied it
+  __shared__ int sm_qtaken_all[kGroups][C::kQBufs];   // consumers that took this query buffer
+  __shared__ int sm_arrived_all[kGroups][C::kFoldBufs];
+  __shared__ int sm_folded_all[kGroups][C::kFoldBufs];
   __shared__ int sm_abort;
 
-  __shared__ int sm_simd[kWaves];
   const int tid = threadIdx.x, lane = tid & 63;
   const int hw_wave = tid >> 6;
+  const int group = hw_wave / kGroupWaves;
+  // role index: consumers 0..kConsumers-1, producer kConsumers
+  const int wave = hw_wave % kGroupWaves == 0 ? kConsumers : hw_wave % kGroupWaves - 1;
   JPT_TR(const unsigned long long tr_start = __builtin_amdgcn_s_memrealtime();)
   JPT_TR(unsigned long long tr_wait = 0; unsigned long long tr_fold = 0; unsigned long long tr_first = 0; unsigned long long tr_t = 0; int tr_tiles = 0;)
-  if (tid < C::kSlots) { sm_filled[tid] = 0; sm_freed[tid] = 0; }
-  if (tid < C::kFoldBufs) { sm_arrived[tid] = 0; sm_folded[tid] = 0; }
-  if (tid == 0) sm_abort = 0;
-  if (lane == 0) sm_simd[hw_wave] = (__builtin_amdgcn_s_getreg(0xF804) >> 4) & 3;  // HW_REG_HW_ID: SIMD_ID
-  __syncthreads();
-  // Roles.  The producer is nearly idle, so the two workgroups sharing a
-  // compute unit should not both park theirs on the same SIMD: pick the wave
-  // that runs on a SIMD derived from the workgroup id (workgroups j and j+32
-  // of an XCD share a unit), if there is one.  `wave` is the role index:
-  // consumers 0..kConsumers-1, producer kConsumers.
-  int producer_wave;
-  {
-    const int j = blockIdx.x >> 3;
-    const int want = (((j >> 5) & 1) << 1) | (j & 1);
-    producer_wave = want % kWaves;
-    for (int w = kWaves - 1; w >= 0; --w)
-      if (sm_simd[w] == want) producer_wave = w;
+  for (int i = tid; i < kGroups * C::kSlots; i += kThreads) {
+    (&sm_filled_all[0][0])[i] = 0;
+    (&sm_freed_all[0][0])[i] = 0;
   }
-  const int wave = hw_wave == producer_wave ? kConsumers : hw_wave - (hw_wave > producer_wave ? 1 : 0);
+  if (tid < kGroups * C::kFoldBufs) {
+    (&sm_arrived_all[0][0])[tid] = 0;
+    (&sm_folded_all[0][0])[tid] = 0;
+  }
+  if (tid < kGroups * C::kQBufs) (&sm_qtaken_all[0][0])[tid] = 0;
+  if (tid == 0) sm_abort = 0;
+  __syncthreads();
+  char* const ring = ring_all[group];
+  auto& sm_o = sm_o_all[group];
+  auto& sm_q = sm_q_all[group];
+  auto& sm_m = sm_m_all[group];
+  auto& sm_l = sm_l_all[group];
+  int* const sm_filled = sm_filled_all[group];
+  int* const sm_freed = sm_freed_all[group];
+  int* const sm_qtaken = sm_qtaken_all[group];
+  int* const sm_arrived = sm_arrived_all[group];
+  int* const sm_folded = sm_folded_all[group];
 
   const int R = p.rows;
-  const int G = gridDim.x;  // multiple of 8
+  // The groups of all workgroups are the workers; worker ids of one workgroup
+  // are equal mod 8 when the grid is a multiple of 8.
+  const int G = kGroups * static_cast<int>(gridDim.x);
+  const int worker = static_cast<int>(blockIdx.x) + group * static_cast<int>(gridDim.x);
   const bool has_new = a.new_k != nullptr;
 
-  // Item sequence of this workgroup: virtual ids k*G + j with j running
-  // forwards in even rounds and backwards in odd ones, so that with entries
-  // sorted longest first every workgroup gets a similar total.  Virtual id i
-  // maps to (entry, head) with all heads of an entry on ids of equal i % 8:
-  // workgroup ids go round-robin over the 8 XCDs, so an entry's scales and
-  // page-table row are fetched into one L2 only.
+  // Item sequence of this worker: virtual ids k*G + j with j running forwards
+  // in even rounds and backwards in odd ones, so that with entries sorted
+  // longest first every worker gets a similar total.  Virtual id i maps to
+  // (entry, head) with all heads of an entry on ids of equal i % 8: workgroup
+  // ids go round-robin over the 8 XCDs, so an entry's scales and page-table
+  // row are fetched into one L2 only.
   auto fetch = [&](int k) -> Item {
     Item it;
-    const int j = (k & 1) ? (G - 1 - static_cast<int>(blockIdx.x)) : static_cast<int>(blockIdx.x);
+    const int j = (k & 1) ? (G - 1 - worker) : worker;
     const int i = k * G + j;
     it.valid = i < p.total_items;
     it.slot = it.start = it.count = it.part = it.n_chunks = it.h = 0;
@@ -322,32 +385,75 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     // scales, one load for both rows: float32 - lanes 0..31 k, 32..63 v;
     // bf16 - lanes 0..15 k, 16..31 v (two positions per lane)
     constexpr int kHalf = SCALE == kScaleF32 ? 32 : 16;
-    const char* scale_lane = nullptr;
+    constexpr int kEs = SCALE == kScaleF32 ? 4 : 2;
+    const char *scale_lane = nullptr, *new_scale_lane = nullptr;
     if (SCALE) {
       const bool is_v = lane >= kHalf;
       scale_lane = static_cast<const char*>(is_v ? a.v_scale : a.k_scale) + (lane - (is_v ? kHalf : 0)) * 4;
+      // the new token's two float32 scales, each repeated over its 32 lanes
+      if (SCALE == kScaleF32 && has_new)
+        new_scale_lane = static_cast<const char*>(is_v ? a.new_v_scale : a.new_k_scale);
     }
-    constexpr int kEs = SCALE == kScaleF32 ? 4 : 2;
+    const int q_loads = (R + 3) / 4;  // load instructions for an item's query rows
 
-    int issued = 0, signalled = 0;
+    int issued = 0, signalled = 0;        // tiles
+    int loads_issued = 0;                 // load instructions, all tiles and query rows
+    int sig_base = 0;                     // loads issued up to the last signalled tile
+    uint64_t carries_q = 0;               // bit t % 64: query rows were loaded just before tile t
     int fill_slot = 0, fill_round = 0;    // issued % kSlots, issued / kSlots
     int sig_slot = 0, sig_round = 1;      // signalled % kSlots, signalled / kSlots + 1
     // Hands every tile that has landed to the consumers.  Loads complete in
     // order, so with `out` loads still counted as outstanding (the wave's own
-    // vector-memory counter, read without waiting) all tiles but the newest
-    // ceil(out / loads-per-tile) are complete.
+    // vector-memory counter, read without waiting) the first
+    // loads_issued - out loads are complete.
     auto signal_landed = [&]() {
       const uint32_t ib = __builtin_amdgcn_s_getreg(0xF807);  // HW_REG_IB_STS, all 32 bits
       const int out = static_cast<int>((ib & 0xF) | (((ib >> 22) & 0x3) << 4));
-      const int landed = issued - (out + C::kLoadsPerTile - 1) / C::kLoadsPerTile;
-      while (signalled < landed) {
+      const int done = loads_issued - out;
+      while (signalled < issued) {
+        const int need = sig_base + C::kLoadsPerTile + (((carries_q >> (signalled & 63)) & 1) ? q_loads : 0);
+        if (done < need) break;
         if (lane == 0) lds_poke(&sm_filled[sig_slot], sig_round);
+        sig_base = need;
+        carries_q &= ~(1ull << (signalled & 63));
         ++signalled;
         if (++sig_slot == C::kSlots) { sig_slot = 0; ++sig_round; }
       }
     };
+    // Bounded wait with hand-overs going on; false = abort.
+    auto wait_counter = [&](int* counter, int needed) -> bool {
+      for (int spins = 0;; ++spins) {
+        signal_landed();
+        if (lds_peek(counter) >= needed) return true;
+        if (spins > kSpinLimit || lds_peek(&sm_abort)) {
+          lds_poke(&sm_abort, 1);
+          __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+          return false;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+    };
+    // Query rows of the `seq`-th item that has tiles into their buffer: piece
+    // 64j + lane of the item's R contiguous 256-byte rows.
+    auto issue_q = [&](const Item& it, int seq) -> bool {
+      const int buf = seq % C::kQBufs;
+      if (!wait_counter(&sm_qtaken[buf], kConsumers * (seq / C::kQBufs))) return false;
+      const char* qrow = static_cast<const char*>(a.q) +
+          ((static_cast<int64_t>(it.slot) * a.q_heads + it.h * p.rep) * a.q_rows) * (kD * 2);
+      char* dst = reinterpret_cast<char*>(&sm_q[buf][0][0]);
+      for (int j = 0; j < q_loads; ++j) {
+        const int piece = 64 * j + lane;
+        if (piece < R * 16)
+          __builtin_amdgcn_global_load_lds((global_ptr)(qrow + piece * 16), (lds_ptr)(dst + j * 1024), 16, 0, 0);
+      }
+      loads_issued += q_loads;
+      carries_q |= 1ull << (issued & 63);
+      return true;
+    };
+
     Item cur = fetch(0);
     Item nxt = fetch(1);
+    int q_seq = 0;  // items with tiles so far: only those have their query rows staged
     for (int k = 0; cur.valid; ++k) {
       const Item nxt2 = fetch(k + 2);  // entries are read two items ahead of their use
       const int hs = a.scale_heads == 1 ? 0 : cur.h;
@@ -367,11 +473,19 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       for (int ti = 0; ti < nt; ++ti) {
         const bool is_new = ti >= n_cache;
         int valid = 1;  // the new token: every row of the tile is that one token
+        const char* sc_src = scale_lane;
         if (is_new) {
           const int64_t row = static_cast<int64_t>(cur.slot) * a.kv_heads + cur.h;
           kt = static_cast<const char*>(a.new_k) + row * C::kRowBytes;
           vt = static_cast<const char*>(a.new_v) + row * C::kRowBytes;
-          srow = 0;  // its scales are read by the consumers; load the tensors' heads
+          // float32 scales of the new token come through the ring like any
+          // tile's; bf16 ones are read by the consumer, and the tile loads the
+          // head of the scale tensors only to keep its load count
+          srow = 0;
+          if (SCALE == kScaleF32) {
+            sc_src = new_scale_lane;
+            srow = static_cast<int64_t>(cur.slot) * a.scale_heads + hs;
+          }
         } else {
           const int t0 = cur.start + ti * kTile;
           valid = min(kTile, cur.start + cur.count - t0);
@@ -386,19 +500,13 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
             page = load_uniform(a.page_table + (static_cast<int64_t>(cur.slot) * a.max_pages + tn / a.page_size));
           }
         }
+        // an item's query rows travel ahead of its first tile: loads complete
+        // in order, so they are in LDS when any of its tiles is handed over
+        if (ti == 0 && !issue_q(cur, q_seq++)) return;
         // wait for the slot's previous tile to be taken, handing over landed
         // tiles meanwhile
         JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
-        for (int spins = 0;; ++spins) {
-          signal_landed();
-          if (lds_peek(&sm_freed[fill_slot]) >= fill_round) break;
-          if (spins > kSpinLimit || lds_peek(&sm_abort)) {
-            lds_poke(&sm_abort, 1);
-            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-            return;
-          }
-          __builtin_amdgcn_s_sleep(1);
-        }
+        if (!wait_counter(&sm_freed[fill_slot], fill_round)) return;
         JPT_TR(tr_wait += __builtin_amdgcn_s_memrealtime() - tr_t; if (!tr_first) tr_first = __builtin_amdgcn_s_memrealtime() - tr_start;)
         char* slot = ring + fill_slot * C::kSlotBytes;
 #pragma unroll
@@ -410,7 +518,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         char* side = slot + 2 * C::kTileBytes;
         if (SCALE) {
           if (lane < 2 * kHalf)
-            __builtin_amdgcn_global_load_lds((global_ptr)(scale_lane + srow * kEs), (lds_ptr)side, 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((global_ptr)(sc_src + srow * kEs), (lds_ptr)side, 4, 0, 0);
         }
         if (MASK) {
           const float* src = static_cast<const float*>(a.mask) + cur.slot * a.mask_stride_b + (is_new ? 0 : cur.start + ti * kTile);
@@ -418,6 +526,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
             __builtin_amdgcn_global_load_lds((global_ptr)(src + lane), (lds_ptr)(side + 256), 4, 0, 0);
         }
         ++issued;
+        loads_issued += C::kLoadsPerTile;
         if (++fill_slot == C::kSlots) { fill_slot = 0; ++fill_round; }
         if (!PAGED) {
           kt += kTile * C::kRowBytes;
@@ -438,9 +547,9 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       __builtin_amdgcn_s_sleep(1);
     }
     JPT_TR(if (p.trace && lane == 0) {
-      unsigned long long* o = p.trace + (static_cast<size_t>(blockIdx.x) * kWaves + wave) * 8;
+      unsigned long long* o = p.trace + (static_cast<size_t>(blockIdx.x) * kWaves + hw_wave) * 8;
       o[0] = issued; o[1] = tr_wait; o[2] = 0; o[3] = __builtin_amdgcn_s_memrealtime() - tr_start;
-      o[4] = tr_start; o[5] = 0; o[6] = tr_first; o[7] = sm_simd[hw_wave];
+      o[4] = tr_start; o[5] = 0; o[6] = tr_first; o[7] = (__builtin_amdgcn_s_getreg(0xF804) >> 4) & 3;
     })
     return;
   }
@@ -451,83 +560,83 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
 #pragma unroll
   for (int i = 0; i < 8; ++i) pos[i] = 4 * g + (i & 3) + 16 * (i >> 2);
 
-  // Q^T operand: lane (r, g) holds q[row r][32g + 8kk + i], zero for r >= R
-  auto load_q = [&](bf16x8* qop, const Item& it) {
-    const char* qrow = static_cast<const char*>(a.q) +
-        ((static_cast<int64_t>(it.slot) * a.q_heads + it.h * p.rep) * a.q_rows + r) * (kD * 2);
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      uint4 u = make_uint4(0, 0, 0, 0);
-      if (r < R) u = *reinterpret_cast<const uint4*>(qrow + (32 * g + 8 * kk) * 2);
-      qop[kk] = __builtin_bit_cast(bf16x8, u);
-    }
-  };
-
+  using T = Tile<KV>;
+  using Op = typename T::Op;
   const float c2 = a.sm_scale * kLog2e;
-  bf16x8 qop[4];
+  Op qop[4];                // Q^T operand: lane (r, g) holds q[row r][32g + 8kk + i], zero for r >= R
+  float c2_row = c2;        // c2 times the power of two taken out of the row's q (int8 codes only)
+  f32x4 s_init = {0.f, 0.f, 0.f, 0.f};  // score accumulators start here: minus the bias term of the row
   f32x4 acc[8];             // O^T tile j: acc[j][i] = o[row r][32g + 8i + j]
+  f32x4 accw = {0.f, 0.f, 0.f, 0.f};    // sum of the weights fed to the second MFMA (int8 codes only)
   float m_run = -INFINITY;  // log2 units, same in the four lanes of a row
   float l_run = 0.f;        // this lane's share of the row sum
 
-  // Takes tile number `t` of the workgroup's stream out of the ring and
-  // accumulates it; `valid` positions of the tile count.
+  // Takes tile number `t` of the group's stream out of the ring and
+  // accumulates it; `valid` positions of the tile count (all of them when
+  // `full_tag` says so).
   int cur_slot = 0, cur_h = 0;  // of the item being consumed
-  auto consume_tile = [&](int t, int valid, bool is_new) -> bool {
+  auto consume_tile = [&](int t, int valid, bool is_new, auto full_tag) -> bool {
+    constexpr bool FULL = decltype(full_tag)::value;
     const int s = t % C::kSlots;
     JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
     if (!wait_for(&sm_filled[s], t / C::kSlots + 1)) return false;
     JPT_TR(tr_wait += __builtin_amdgcn_s_memrealtime() - tr_t; ++tr_tiles; if (!tr_first) tr_first = __builtin_amdgcn_s_memrealtime() - tr_start;)
     const char* slot = ring + s * C::kSlotBytes;
     const char* side = slot + 2 * C::kTileBytes;
-    Tile<KV> tile;
+    T tile;
     tile.read(slot, slot + C::kTileBytes, r, g, pos);
+    // the lane's positions are 4g..4g+3 and 16+4g..16+4g+3
     float ks[8], vs[8], mk[8];
-    if (SCALE && is_new) {
+    if (SCALE == kScaleF32) {
+      const float4* sk = reinterpret_cast<const float4*>(side);
+      const float4 k0 = sk[g], k1 = sk[4 + g], v0 = sk[8 + g], v1 = sk[12 + g];
+      ks[0] = k0.x; ks[1] = k0.y; ks[2] = k0.z; ks[3] = k0.w; ks[4] = k1.x; ks[5] = k1.y; ks[6] = k1.z; ks[7] = k1.w;
+      vs[0] = v0.x; vs[1] = v0.y; vs[2] = v0.z; vs[3] = v0.w; vs[4] = v1.x; vs[5] = v1.y; vs[6] = v1.z; vs[7] = v1.w;
+    } else if (SCALE == kScaleBF16 && is_new) {
       const int64_t si = static_cast<int64_t>(cur_slot) * a.scale_heads + (a.scale_heads == 1 ? 0 : cur_h);
-      const float nks = load_as_f32(a.new_k_scale, si, SCALE == kScaleF32 ? JPT_F32 : JPT_BF16);
-      const float nvs = load_as_f32(a.new_v_scale, si, SCALE == kScaleF32 ? JPT_F32 : JPT_BF16);
+      const float nks = load_as_f32(a.new_k_scale, si, JPT_BF16);
+      const float nvs = load_as_f32(a.new_v_scale, si, JPT_BF16);
 #pragma unroll
       for (int i = 0; i < 8; ++i) { ks[i] = nks; vs[i] = nvs; }
-    } else if (SCALE == kScaleF32) {
-      const float* sk = reinterpret_cast<const float*>(side);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        ks[i] = sk[pos[i]];
-        vs[i] = sk[32 + pos[i]];
-      }
     } else if (SCALE == kScaleBF16) {
-      const uint16_t* sk = reinterpret_cast<const uint16_t*>(side);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        ks[i] = bf16_bits_to_f32(sk[pos[i]]);
-        vs[i] = bf16_bits_to_f32(sk[32 + pos[i]]);
-      }
+      const uint2* sk = reinterpret_cast<const uint2*>(side);
+      const uint2 k0 = sk[g], k1 = sk[4 + g], v0 = sk[8 + g], v1 = sk[12 + g];
+      ks[0] = __uint_as_float(k0.x << 16); ks[1] = __uint_as_float(k0.x & 0xffff0000u);
+      ks[2] = __uint_as_float(k0.y << 16); ks[3] = __uint_as_float(k0.y & 0xffff0000u);
+      ks[4] = __uint_as_float(k1.x << 16); ks[5] = __uint_as_float(k1.x & 0xffff0000u);
+      ks[6] = __uint_as_float(k1.y << 16); ks[7] = __uint_as_float(k1.y & 0xffff0000u);
+      vs[0] = __uint_as_float(v0.x << 16); vs[1] = __uint_as_float(v0.x & 0xffff0000u);
+      vs[2] = __uint_as_float(v0.y << 16); vs[3] = __uint_as_float(v0.y & 0xffff0000u);
+      vs[4] = __uint_as_float(v1.x << 16); vs[5] = __uint_as_float(v1.x & 0xffff0000u);
+      vs[6] = __uint_as_float(v1.y << 16); vs[7] = __uint_as_float(v1.y & 0xffff0000u);
     }
     if (MASK) {
-      const float* smk = reinterpret_cast<const float*>(side + 256);
+      const float4* smk = reinterpret_cast<const float4*>(side + 256);
+      const float4 m0 = smk[g], m1 = smk[4 + g];
+      mk[0] = m0.x; mk[1] = m0.y; mk[2] = m0.z; mk[3] = m0.w; mk[4] = m1.x; mk[5] = m1.y; mk[6] = m1.z; mk[7] = m1.w;
+      if (is_new) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) mk[i] = is_new ? 0.f : smk[pos[i]];
+        for (int i = 0; i < 8; ++i) mk[i] = 0.f;
+      }
     }
     // the registers hold the tile: hand the slot back (the release waits for
     // the LDS reads above)
     if (lane == 0)
       __hip_atomic_fetch_add(&sm_freed[s], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
 
-    f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+    f32x4 sa = s_init, sb = s_init;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-      sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tile.k_op(false, kk), qop[kk], sa, 0, 0, 0);
-      sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tile.k_op(true, kk), qop[kk], sb, 0, 0, 0);
+      sa = T::mfma(tile.k_op(false, kk), qop[kk], sa);
+      sb = T::mfma(tile.k_op(true, kk), qop[kk], sb);
     }
     float sc[8];
-    bool live[8];
     float tmax = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      float x = (i < 4 ? sa[i] : sb[i - 4]) * (SCALE ? ks[i] * c2 : c2);
+      float x = (i < 4 ? sa[i] : sb[i - 4]) * (SCALE ? ks[i] * c2_row : c2_row);
       if (MASK) x += mk[i] * kLog2e;
-      live[i] = pos[i] < valid && x == x;  // NaN scores attend nothing
-      x = live[i] ? x : -INFINITY;
+      if (!FULL) x = pos[i] < valid ? x : -INFINITY;
       sc[i] = x;
       tmax = fmaxf(tmax, x);
     }
@@ -541,23 +650,25 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     for (int i = 0; i < 8; ++i) {
       const float pr = fast_exp2(sc[i] - m_use);
       psum += pr;
-      w[i] = SCALE ? (live[i] ? pr * vs[i] : 0.f) : pr;
+      // a position that does not count has weight 0 whatever its scale holds
+      w[i] = SCALE ? ((FULL || pos[i] < valid) ? pr * vs[i] : 0.f) : pr;
     }
     l_run = l_run * alpha + psum;
     m_run = m_new;
-    if (__any(alpha != 1.f)) {
+    if (__any(alpha != 1.f)) {  // rare once the running maximum has settled
+      asm volatile("" ::: "memory");  // keeps the compiler from running this speculatively
 #pragma unroll
       for (int j = 0; j < 8; ++j) acc[j] *= alpha;
+      if (T::kBias != 0.f) accw *= alpha;
     }
-    const bf16x8 pop = as_op(pack_bf16(w[0], w[1]), pack_bf16(w[2], w[3]),
-                             pack_bf16(w[4], w[5]), pack_bf16(w[6], w[7]));
+    const Op pop = as_op<Op>(T::pack(w[0], w[1]), T::pack(w[2], w[3]), T::pack(w[4], w[5]), T::pack(w[6], w[7]));
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-      acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tile.v_op(j), pop, acc[j], 0, 0, 0);
+    for (int j = 0; j < 8; ++j) acc[j] = T::mfma(tile.v_op(j), pop, acc[j]);
+    if (T::kBias != 0.f) accw = T::mfma(T::ones(), pop, accw);
     return true;
   };
 
-  // Delivers the wave's part of item number `seq` of this workgroup; the last
+  // Delivers the wave's part of item number `seq` of this group; the last
   // consumer to arrive folds the parts and writes the slot's output (one
   // chunk) or parks the chunk's partial (several).
   auto finish_item = [&](const Item& it, int seq) -> bool {
@@ -567,10 +678,11 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     float l_row = l_run + __shfl_xor(l_run, 16);
     l_row += __shfl_xor(l_row, 32);
     if (r < R) {
+      const float bias = T::kBias * accw[0];  // every element of accw is the row's weight sum
 #pragma unroll
       for (int j = 0; j < 8; ++j)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) sm_o[buf][wave][r][o_col(32 * g + 8 * i + j)] = acc[j][i];
+        for (int i = 0; i < 4; ++i) sm_o[buf][wave][r][o_col(32 * g + 8 * i + j)] = acc[j][i] - bias;
       if (g == 0) {
         sm_m[buf][wave][r] = m_run;
         sm_l[buf][wave][r] = l_row;
@@ -631,31 +743,92 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   Item cur = fetch(0);
   if (!cur.valid) return;
   Item nxt = fetch(1);
-  int base = 0;  // stream number of the current item's tile 0
+  int base = 0;   // stream number of the current item's tile 0
+  int q_seq = 0;  // items with tiles so far
   for (int k = 0;; ++k) {
     const Item nxt2 = fetch(k + 2);
-    load_q(qop, cur);
     const int n_cache = cache_tiles(cur), nt = item_tiles(cur);
+    if (nt > 0) {
+      // query rows: staged by the producer ahead of the item's first tile
+      if (!wait_for(&sm_filled[base % C::kSlots], base / C::kSlots + 1)) return;
+      const int qb = q_seq++ % C::kQBufs;
+      uint4 u[4];
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        u[kk] = make_uint4(0, 0, 0, 0);
+        if (r < R) u[kk] = *reinterpret_cast<const uint4*>(&sm_q[qb][r][32 * g + 8 * kk]);
+      }
+      if (T::kBias == 0.f) {
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) qop[kk] = __builtin_bit_cast(Op, u[kk]);
+      } else {
+        // float16 operand: the row is scaled by a power of two that puts its
+        // largest magnitude in [2^13, 2^14) (exact; the power goes into
+        // c2_row), and the bias term 1152 * sum(q) of the row is summed up
+        float f[32];
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          const uint32_t wds[4] = {u[kk].x, u[kk].y, u[kk].z, u[kk].w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            f[8 * kk + 2 * i] = __uint_as_float(wds[i] << 16);
+            f[8 * kk + 2 * i + 1] = __uint_as_float(wds[i] & 0xffff0000u);
+          }
+        }
+        float amax = 0.f;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(f[i]));
+        amax = fmaxf(amax, __shfl_xor(amax, 16));
+        amax = fmaxf(amax, __shfl_xor(amax, 32));
+        int e = 0;
+        if (amax > 0.f && amax < INFINITY) frexpf(amax, &e);
+        e = max(e, -100);
+        const float up = ldexpf(1.f, 14 - e);
+        c2_row = c2 * ldexpf(1.f, e - 14);
+        float qs = 0.f;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+          f[i] *= up;
+          qs += f[i];
+        }
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+          qop[kk] = as_op<Op>(pack_f16(f[8 * kk], f[8 * kk + 1]), pack_f16(f[8 * kk + 2], f[8 * kk + 3]),
+                              pack_f16(f[8 * kk + 4], f[8 * kk + 5]), pack_f16(f[8 * kk + 6], f[8 * kk + 7]));
+        qs += __shfl_xor(qs, 16);
+        qs += __shfl_xor(qs, 32);
+        const float ncq = -T::kBias * qs;
+        s_init = f32x4{ncq, ncq, ncq, ncq};
+      }
+      // taken (the release waits for the reads above)
+      if (lane == 0)
+        __hip_atomic_fetch_add(&sm_qtaken[qb], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
     cur_slot = cur.slot;
     cur_h = cur.h;
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    accw = f32x4{0.f, 0.f, 0.f, 0.f};
     m_run = -INFINITY;
     l_run = 0.f;
     // this consumer's tiles: stream numbers congruent to its index
     for (int ti = (wave + kConsumers - base % kConsumers) % kConsumers; ti < nt; ti += kConsumers) {
       const bool is_new = ti >= n_cache;
       const int valid = is_new ? 1 : min(kTile, cur.count - ti * kTile);
-      if (!consume_tile(base + ti, valid, is_new)) return;
+      if (valid == kTile) {
+        if (!consume_tile(base + ti, valid, false, std::true_type{})) return;
+      } else {
+        if (!consume_tile(base + ti, valid, is_new, std::false_type{})) return;
+      }
     }
     JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
     if (!finish_item(cur, k)) return;
     JPT_TR(tr_fold += __builtin_amdgcn_s_memrealtime() - tr_t;)
     if (!nxt.valid) {
       JPT_TR(if (p.trace && lane == 0) {
-        unsigned long long* o = p.trace + (static_cast<size_t>(blockIdx.x) * kWaves + wave) * 8;
+        unsigned long long* o = p.trace + (static_cast<size_t>(blockIdx.x) * kWaves + hw_wave) * 8;
         o[0] = tr_tiles; o[1] = tr_wait; o[2] = tr_fold; o[3] = __builtin_amdgcn_s_memrealtime() - tr_start;
-        o[4] = tr_start; o[5] = k + 1; o[6] = tr_first; o[7] = sm_simd[hw_wave];
+        o[4] = tr_start; o[5] = k + 1; o[6] = tr_first; o[7] = (__builtin_amdgcn_s_getreg(0xF804) >> 4) & 3;
       })
       break;
     }
@@ -665,8 +838,10 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   }
 }
 
+// `workers` groups are wanted; a workgroup holds kGroups of them.
 template <typename KV, bool PAGED, int SCALE, bool MASK>
-void launch_rows(const FastParams& p, unsigned blocks, hipStream_t stream) {
+void launch_rows(const FastParams& p, unsigned workers, hipStream_t stream) {
+  const unsigned blocks = workers / kGroups > 0 ? workers / kGroups : 1;
   if (p.rows <= 4)
     hipLaunchKernelGGL((attn_decode_kernel<KV, PAGED, SCALE, MASK, 4>), dim3(blocks), dim3(kThreads), 0, stream, p);
   else if (p.rows <= 8)
