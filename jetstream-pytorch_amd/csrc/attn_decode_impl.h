@@ -70,6 +70,7 @@ constexpr int kSideBytes = 512;     // ks | vs | mask, 128 bytes each at most
 constexpr int kOStride = 140;       // padded LDS row of 128 outputs
 constexpr int kLdsBudget = 160 * 1024 / kGroups - 512;  // per group; one workgroup per compute unit
 constexpr int kSpinLimit = 1 << 18;  // tens of milliseconds
+constexpr int kListedItems = 64;     // a worker's first items, read into LDS at start
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -96,8 +97,8 @@ struct Config {
   static constexpr int kQLoadsMax = (RC + 3) / 4;  // 1 KiB (four rows) a load
   static constexpr int kFoldPart = kConsumers * RC * (kOStride + 2) * 4;
   // ring slots: every one may hold a tile in flight, and the wave's load
-  // counter counts to 63
-  static constexpr int kSlotsByCount = (63 - kQLoadsMax) / kLoadsPerTile;
+  // counter counts to 63 (the producer checks the room before each issue)
+  static constexpr int kSlotsByCount = 63 / kLoadsPerTile;
   static constexpr int kSlotsWith2 = (kLdsBudget - kQBytes - 2 * kFoldPart) / kSlotBytes;
   static constexpr int kEnough = kSlotsByCount < 5 ? kSlotsByCount : 5;
   static constexpr int kFoldBufs = kSlotsWith2 >= kEnough ? 2 : 1;
@@ -115,6 +116,13 @@ __device__ __forceinline__ int lds_peek(const int* p) {
   const uint32_t addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_int_ptr)p));
   int v;
   asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
+  return v;
+}
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+__device__ __forceinline__ i32x4 lds_peek4(const int* p) {
+  const uint32_t addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_int_ptr)p));
+  i32x4 v;
+  asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
   return v;
 }
 __device__ __forceinline__ void lds_poke(int* p, int v) {
@@ -287,6 +295,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   __shared__ int sm_arrived_all[kGroups][C::kFoldBufs];
   __shared__ int sm_folded_all[kGroups][C::kFoldBufs];
   __shared__ int sm_abort;
+  __shared__ __attribute__((aligned(16))) int sm_items_all[kGroups][kListedItems][8];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int hw_wave = tid >> 6;
@@ -305,7 +314,32 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   }
   if (tid < kGroups * C::kQBufs) (&sm_qtaken_all[0][0])[tid] = 0;
   if (tid == 0) sm_abort = 0;
-  __syncthreads();
+
+  const int R = p.rows;
+  // The groups of all workgroups are the workers; worker ids of one workgroup
+  // are equal mod 8 when the grid is a multiple of 8.
+  const int G = kGroups * static_cast<int>(gridDim.x);
+  const int worker = static_cast<int>(blockIdx.x) + group * static_cast<int>(gridDim.x);
+  const int n_rounds = (p.total_items + G - 1) / G;
+  const bool has_new = a.new_k != nullptr;
+
+  // Item of round k of this worker: virtual ids k*G + j with j running forwards
+  // in even rounds and backwards in odd ones, so that with entries sorted
+  // longest first every worker gets a similar total.  Virtual id i maps to
+  // (entry, head) with all heads of an entry on ids of equal i % 8: workgroup
+  // ids go round-robin over the 8 XCDs, so an entry's scales and page-table
+  // row are fetched into one L2 only.  Unused entries give invalid items.
+  auto item_index = [&](int k, int* entry, int* h) -> bool {
+    const int j = (k & 1) ? (G - 1 - worker) : worker;
+    const int i = k * G + j;
+    const int m = i >> 3;
+    *entry = (m / a.kv_heads) * 8 + (i & 7);
+    *h = m % a.kv_heads;
+    return k < n_rounds && i < p.total_items;
+  };
+  // The first kListedItems rounds are read here, all at once, into LDS (one
+  // memory latency for the lot, and none inside the stream); later rounds, which
+  // only very large batches have, are read when they are reached.
   char* const ring = ring_all[group];
   auto& sm_o = sm_o_all[group];
   auto& sm_q = sm_q_all[group];
@@ -316,30 +350,40 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   int* const sm_qtaken = sm_qtaken_all[group];
   int* const sm_arrived = sm_arrived_all[group];
   int* const sm_folded = sm_folded_all[group];
-
-  const int R = p.rows;
-  // The groups of all workgroups are the workers; worker ids of one workgroup
-  // are equal mod 8 when the grid is a multiple of 8.
-  const int G = kGroups * static_cast<int>(gridDim.x);
-  const int worker = static_cast<int>(blockIdx.x) + group * static_cast<int>(gridDim.x);
-  const bool has_new = a.new_k != nullptr;
-
-  // Item sequence of this worker: virtual ids k*G + j with j running forwards
-  // in even rounds and backwards in odd ones, so that with entries sorted
-  // longest first every worker gets a similar total.  Virtual id i maps to
-  // (entry, head) with all heads of an entry on ids of equal i % 8: workgroup
-  // ids go round-robin over the 8 XCDs, so an entry's scales and page-table
-  // row are fetched into one L2 only.
-  auto fetch = [&](int k) -> Item {
+  int (*const sm_items)[8] = sm_items_all[group];
+  if (wave == kConsumers) {
+    int entry, h;
+    const bool in_range = item_index(lane, &entry, &h);
+    int4 e0 = make_int4(-1, 0, 0, 0), e1 = make_int4(0, 0, 0, 0);
+    if (in_range) {
+      const int4* en = reinterpret_cast<const int4*>(p.entries + entry);
+      e0 = en[0];
+      e1 = en[1];
+    }
+    // slot, start, count, part | n_chunks, head, valid
+    *reinterpret_cast<int4*>(&sm_items[lane][0]) = e0;
+    *reinterpret_cast<int4*>(&sm_items[lane][4]) = make_int4(e1.x, h, e0.x >= 0 ? 1 : 0, 0);
+  }
+  __syncthreads();
+  auto unpack_item = [&](int4 e0, int4 e1) -> Item {
     Item it;
-    const int j = (k & 1) ? (G - 1 - worker) : worker;
-    const int i = k * G + j;
-    it.valid = i < p.total_items;
+    it.slot = __builtin_amdgcn_readfirstlane(e0.x);
+    it.start = __builtin_amdgcn_readfirstlane(e0.y);
+    it.count = __builtin_amdgcn_readfirstlane(e0.z);
+    it.part = __builtin_amdgcn_readfirstlane(e0.w);
+    it.n_chunks = __builtin_amdgcn_readfirstlane(e1.x);
+    it.h = __builtin_amdgcn_readfirstlane(e1.y);
+    it.valid = __builtin_amdgcn_readfirstlane(e1.z) != 0;
+    return it;
+  };
+  auto fetch = [&](int k) -> Item {  // rounds past the listed ones
+    Item it;
+    int entry, h;
+    it.valid = item_index(k, &entry, &h);
     it.slot = it.start = it.count = it.part = it.n_chunks = it.h = 0;
     if (it.valid) {
-      const int m = i >> 3;
-      const int32_t* en = reinterpret_cast<const int32_t*>(p.entries + ((m / a.kv_heads) * 8 + (i & 7)));
-      it.h = m % a.kv_heads;
+      const int32_t* en = reinterpret_cast<const int32_t*>(p.entries + entry);
+      it.h = h;
       it.slot = load_uniform(en + 0); it.start = load_uniform(en + 1); it.count = load_uniform(en + 2);
       it.part = load_uniform(en + 3); it.n_chunks = load_uniform(en + 4);
       it.valid = it.slot >= 0;
@@ -420,11 +464,12 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         if (++sig_slot == C::kSlots) { sig_slot = 0; ++sig_round; }
       }
     };
-    // Bounded wait with hand-overs going on; false = abort.
-    auto wait_counter = [&](int* counter, int needed) -> bool {
+    // Bounded wait with hand-overs going on; false = abort.  Also waits until
+    // `room` more loads fit under the load counter's limit of 63.
+    auto wait_counter = [&](int* counter, int needed, int room) -> bool {
       for (int spins = 0;; ++spins) {
         signal_landed();
-        if (lds_peek(counter) >= needed) return true;
+        if (loads_issued - sig_base + room <= 63 && lds_peek(counter) >= needed) return true;
         if (spins > kSpinLimit || lds_peek(&sm_abort)) {
           lds_poke(&sm_abort, 1);
           __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
@@ -437,7 +482,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     // 64j + lane of the item's R contiguous 256-byte rows.
     auto issue_q = [&](const Item& it, int seq) -> bool {
       const int buf = seq % C::kQBufs;
-      if (!wait_counter(&sm_qtaken[buf], kConsumers * (seq / C::kQBufs))) return false;
+      if (!wait_counter(&sm_qtaken[buf], kConsumers * (seq / C::kQBufs), q_loads)) return false;
       const char* qrow = static_cast<const char*>(a.q) +
           ((static_cast<int64_t>(it.slot) * a.q_heads + it.h * p.rep) * a.q_rows) * (kD * 2);
       char* dst = reinterpret_cast<char*>(&sm_q[buf][0][0]);
@@ -451,11 +496,16 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       return true;
     };
 
-    Item cur = fetch(0);
-    Item nxt = fetch(1);
     int q_seq = 0;  // items with tiles so far: only those have their query rows staged
-    for (int k = 0; cur.valid; ++k) {
-      const Item nxt2 = fetch(k + 2);  // entries are read two items ahead of their use
+    for (int k = 0; k < n_rounds; ++k) {
+      Item cur;
+      if (k < kListedItems) {
+        const i32x4 e0 = lds_peek4(&sm_items[k][0]), e1 = lds_peek4(&sm_items[k][4]);
+        cur = unpack_item(make_int4(e0[0], e0[1], e0[2], e0[3]), make_int4(e1[0], e1[1], e1[2], e1[3]));
+      } else {
+        cur = fetch(k);
+      }
+      if (!cur.valid) continue;
       const int hs = a.scale_heads == 1 ? 0 : cur.h;
       const int n_cache = cache_tiles(cur), nt = item_tiles(cur);
       // rows of the item's first position in the key/value and scale tensors
@@ -506,7 +556,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         // wait for the slot's previous tile to be taken, handing over landed
         // tiles meanwhile
         JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
-        if (!wait_counter(&sm_freed[fill_slot], fill_round)) return;
+        if (!wait_counter(&sm_freed[fill_slot], fill_round, C::kLoadsPerTile)) return;
         JPT_TR(tr_wait += __builtin_amdgcn_s_memrealtime() - tr_t; if (!tr_first) tr_first = __builtin_amdgcn_s_memrealtime() - tr_start;)
         char* slot = ring + fill_slot * C::kSlotBytes;
 #pragma unroll
@@ -534,8 +584,6 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
           srow += kTile;
         }
       }
-      cur = nxt;
-      nxt = nxt2;
     }
     for (int spins = 0; signalled < issued; ++spins) {
       signal_landed();
@@ -740,13 +788,19 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     return true;
   };
 
-  Item cur = fetch(0);
-  if (!cur.valid) return;
-  Item nxt = fetch(1);
   int base = 0;   // stream number of the current item's tile 0
   int q_seq = 0;  // items with tiles so far
-  for (int k = 0;; ++k) {
-    const Item nxt2 = fetch(k + 2);
+  int seq = 0;    // valid items so far
+  for (int k = 0; k < n_rounds; ++k) {
+    Item cur;
+    if (k < kListedItems) {
+      const int4 e0 = *reinterpret_cast<const int4*>(&sm_items[k][0]);
+      const int4 e1 = *reinterpret_cast<const int4*>(&sm_items[k][4]);
+      cur = unpack_item(e0, e1);
+    } else {
+      cur = fetch(k);
+    }
+    if (!cur.valid) continue;
     const int n_cache = cache_tiles(cur), nt = item_tiles(cur);
     if (nt > 0) {
       // query rows: staged by the producer ahead of the item's first tile
@@ -822,20 +876,15 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       }
     }
     JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
-    if (!finish_item(cur, k)) return;
+    if (!finish_item(cur, seq++)) return;
     JPT_TR(tr_fold += __builtin_amdgcn_s_memrealtime() - tr_t;)
-    if (!nxt.valid) {
-      JPT_TR(if (p.trace && lane == 0) {
-        unsigned long long* o = p.trace + (static_cast<size_t>(blockIdx.x) * kWaves + hw_wave) * 8;
-        o[0] = tr_tiles; o[1] = tr_wait; o[2] = tr_fold; o[3] = __builtin_amdgcn_s_memrealtime() - tr_start;
-        o[4] = tr_start; o[5] = k + 1; o[6] = tr_first; o[7] = (__builtin_amdgcn_s_getreg(0xF804) >> 4) & 3;
-      })
-      break;
-    }
     base += nt;
-    cur = nxt;
-    nxt = nxt2;
   }
+  JPT_TR(if (p.trace && lane == 0) {
+    unsigned long long* o = p.trace + (static_cast<size_t>(blockIdx.x) * kWaves + hw_wave) * 8;
+    o[0] = tr_tiles; o[1] = tr_wait; o[2] = tr_fold; o[3] = __builtin_amdgcn_s_memrealtime() - tr_start;
+    o[4] = tr_start; o[5] = seq; o[6] = tr_first; o[7] = (__builtin_amdgcn_s_getreg(0xF804) >> 4) & 3;
+  })
 }
 
 // `workers` groups are wanted; a workgroup holds kGroups of them.
