@@ -146,55 +146,64 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
 }
 
 // Folds the partials of every slot that was split into several chunks: one
-// workgroup per (slot, KV head).  The chunk maxima and sums go through LDS
-// first; then thread (row, d) walks the chunks with independent loads, eight
-// in flight.
-__global__ void __launch_bounds__(512) attn_merge_kernel(FastParams p) {
+// workgroup per (slot, KV head), 16 lanes a row, eight consecutive outputs a
+// lane.  A lane loads its share of up to eight chunks - outputs, maxima and
+// sums alike - in one batch of independent loads, so a slot of up to eight
+// chunks costs one memory round trip; longer ones are folded batch by batch.
+constexpr int kMergeBatch = 8;
+__global__ void __launch_bounds__(256) attn_merge_kernel(FastParams p) {
   const jpt_attn_args& a = p.a;
   const int b = blockIdx.x / a.kv_heads, h = blockIdx.x % a.kv_heads;
   const SlotChunks sc = p.slots[b];
-  if (sc.n_chunks <= 1) return;
-  __shared__ float s_mc[kMaxChunksPerSlot * kMaxRows];  // [chunk][row]
-  __shared__ float s_lc[kMaxChunksPerSlot * kMaxRows];
-  __shared__ float s_m[kMaxRows], s_l[kMaxRows];
   const int R = p.rows, n = sc.n_chunks;
-  const int tid = threadIdx.x;
+  const int row = threadIdx.x >> 4, d0 = 8 * (threadIdx.x & 15);
+  if (n <= 1 || row >= R) return;
   const int64_t rec = static_cast<int64_t>(R) * kPartFloats;
-  const float* first = p.partials + (static_cast<int64_t>(sc.first_part) * a.kv_heads + h) * rec;
+  const float* base = p.partials + (static_cast<int64_t>(sc.first_part) * a.kv_heads + h) * rec + row * kPartFloats;
   const int64_t step = static_cast<int64_t>(a.kv_heads) * rec;
-  const int64_t q_row0 = (static_cast<int64_t>(b) * a.q_heads + h * p.rep) * a.q_rows;
-  for (int i = tid; i < n * R; i += blockDim.x) {
-    const float* base = first + (i / R) * step + (i % R) * kPartFloats;
-    s_mc[i] = base[kD];
-    s_lc[i] = base[kD + 1];
+  float M = -INFINITY, L = 0.f;
+  float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int c0 = 0; c0 < n; c0 += kMergeBatch) {
+    float4 x[kMergeBatch], y[kMergeBatch];
+    float2 ml[kMergeBatch];
+#pragma unroll
+    for (int c = 0; c < kMergeBatch; ++c) {
+      ml[c] = make_float2(-INFINITY, 0.f);
+      x[c] = y[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (c0 + c < n) {
+        const float* src = base + (c0 + c) * step;
+        ml[c] = *reinterpret_cast<const float2*>(src + kD);
+        x[c] = *reinterpret_cast<const float4*>(src + d0);
+        y[c] = *reinterpret_cast<const float4*>(src + d0 + 4);
+      }
+    }
+    float Mb = M;
+#pragma unroll
+    for (int c = 0; c < kMergeBatch; ++c) Mb = fmaxf(Mb, ml[c].x);
+    const float keep = M == -INFINITY ? 0.f : exp2f(M - Mb);
+    L *= keep;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] *= keep;
+#pragma unroll
+    for (int c = 0; c < kMergeBatch; ++c) {
+      const float f = ml[c].x == -INFINITY ? 0.f : exp2f(ml[c].x - Mb);
+      L += ml[c].y * f;
+      o[0] += x[c].x * f; o[1] += x[c].y * f; o[2] += x[c].z * f; o[3] += x[c].w * f;
+      o[4] += y[c].x * f; o[5] += y[c].y * f; o[6] += y[c].z * f; o[7] += y[c].w * f;
+    }
+    M = Mb;
   }
-  __syncthreads();
-  if (tid < R) {
-    float M = -INFINITY, L = 0.f;
-    for (int c = 0; c < n; ++c) M = fmaxf(M, s_mc[c * R + tid]);
-    for (int c = 0; c < n; ++c) {
-      const float mc = s_mc[c * R + tid];
-      L += mc == -INFINITY ? 0.f : exp2f(mc - M) * s_lc[c * R + tid];
-    }
-    s_m[tid] = M;
-    s_l[tid] = L;
-  }
-  __syncthreads();
-  for (int idx = tid; idx < R * kD; idx += blockDim.x) {
-    const int row = idx / kD, d = idx % kD;
-    const float M = s_m[row], L = s_l[row];
-    const float* col = first + row * kPartFloats + d;
-    float o = 0.f;
-#pragma unroll 8
-    for (int c = 0; c < n; ++c) {
-      const float mc = s_mc[c * R + row];
-      o += col[c * step] * (mc == -INFINITY ? 0.f : exp2f(mc - M));
-    }
-    static_cast<uint16_t*>(a.out)[(q_row0 + row) * kD + d] = f32_to_bf16_bits(L > 0.f ? o / L : 0.f);
-    if (d == 0) {
-      if (a.out_max) a.out_max[q_row0 + row] = M * kLn2;
-      if (a.out_denom) a.out_denom[q_row0 + row] = L;
-    }
+  const int64_t q_row = (static_cast<int64_t>(b) * a.q_heads + h * p.rep) * a.q_rows + row;
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  uint4 packed;
+  packed.x = f32_to_bf16_bits(o[0] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[1] * inv)) << 16);
+  packed.y = f32_to_bf16_bits(o[2] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[3] * inv)) << 16);
+  packed.z = f32_to_bf16_bits(o[4] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[5] * inv)) << 16);
+  packed.w = f32_to_bf16_bits(o[6] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[7] * inv)) << 16);
+  *reinterpret_cast<uint4*>(static_cast<uint16_t*>(a.out) + q_row * kD + d0) = packed;
+  if (d0 == 0) {
+    if (a.out_max) a.out_max[q_row] = M * kLn2;
+    if (a.out_denom) a.out_denom[q_row] = L;
   }
 }
 
@@ -273,7 +282,7 @@ int32_t attn_fast_launch(const jpt_attn_args& a, AttnMode mode, hipStream_t stre
   else decode::launch_decode_bf16(p, mode == kPaged, blocks, stream);
   int32_t st = launch_status("attn_decode_kernel");
   if (st != JPT_OK) return st;
-  hipLaunchKernelGGL(attn_merge_kernel, dim3(a.batch * a.kv_heads), dim3(512), 0, stream, p);
+  hipLaunchKernelGGL(attn_merge_kernel, dim3(a.batch * a.kv_heads), dim3(256), 0, stream, p);
   return launch_status("attn_merge_kernel");
 }
 

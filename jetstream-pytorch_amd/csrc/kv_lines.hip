@@ -161,6 +161,95 @@ __global__ void __launch_bounds__(256) quant_append_kernel(QuantParams p) {
   }
 }
 
+// The same computation for the common shape: bf16 input, four elements a
+// thread kept in registers between the absmax pass and the quantise pass
+// (heads * dim == 4 * blockDim), codes stored four at a time.
+template <bool BF16_MATH>
+__global__ void __launch_bounds__(256) quant_append_vec_kernel(QuantParams p) {
+  const jpt_quant_append_args& a = p.a;
+  const bool paged = p.indices != nullptr;
+  const int tok = blockIdx.x;
+  const int b = paged ? p.indices[2 * p.n_active + tok] : tok;
+  const bool is_v = blockIdx.y == 1;
+  const uint16_t* src = static_cast<const uint16_t*>(is_v ? a.new_v : a.new_k);
+  int8_t* cache = static_cast<int8_t*>(is_v ? a.cache_v : a.cache_k);
+  void* scale_out = is_v ? a.v_scale : a.k_scale;
+  int8_t* stash = static_cast<int8_t*>(is_v ? a.out_v : a.out_k);
+  void* stash_scale = is_v ? a.out_v_scale : a.out_k_scale;
+  const int H = a.heads, D = a.dim, HD = H * D;
+  const int groups = a.scale_heads;  // 1 or H
+  const int i0 = 4 * threadIdx.x;    // this thread's elements i0 .. i0 + 3, all of head h
+  const int h = i0 / D, d = i0 - h * D;
+  const int64_t src_base = static_cast<int64_t>(b) * HD;
+
+  // destination of this token's rows (read early: the loads overlap)
+  int at, page = 0;
+  bool write_cache = cache != nullptr;
+  if (paged) {
+    page = p.indices[tok];
+    at = p.indices[p.n_active + tok] % p.page_size;
+    write_cache = write_cache && page >= 0 && page < p.total_pages;
+  } else {
+    at = a.pos ? a.pos[a.pos_count == 1 ? 0 : b] : 0;
+    write_cache = write_cache && at >= 0 && at < a.seq;
+  }
+  const uint2 raw = *reinterpret_cast<const uint2*>(src + src_base + i0);
+  float x[4] = {__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
+                __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u)};
+  float m = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
+
+  __shared__ float s_red[64];
+  float amax;
+  if (groups == 1) {
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    amax = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+  } else {
+    // a head's D / 4 threads are consecutive; D / 4 is a power of two <= 64
+    for (int off = D / 8; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    amax = m;
+  }
+  if (a.rounding == JPT_ROUND_RNE) amax = fmaxf(amax, rnd<BF16_MATH>(1e-5f));
+  const float s = rnd<BF16_MATH>(amax / 127.0f);
+
+  int code[4];
+  if (a.rounding == JPT_ROUND_TRUNC) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float q = rnd<BF16_MATH>(x[i] / s);
+      code[i] = (q != q) ? 0 : static_cast<int>(q);  // 0/0 -> 0; cast truncates
+    }
+  } else {
+    const float r = rnd<BF16_MATH>(1.0f / s);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float q = rnd<BF16_MATH>(x[i] * r);
+      code[i] = static_cast<int>(fminf(fmaxf(rintf(q), -128.f), 127.f));
+    }
+  }
+  const uint32_t packed = (static_cast<uint32_t>(code[0]) & 0xffu) | ((static_cast<uint32_t>(code[1]) & 0xffu) << 8) |
+                          ((static_cast<uint32_t>(code[2]) & 0xffu) << 16) | (static_cast<uint32_t>(code[3]) << 24);
+  if (stash) *reinterpret_cast<uint32_t*>(stash + src_base + i0) = packed;
+  if (write_cache) {
+    const int64_t row = paged
+        ? (static_cast<int64_t>(h) * p.total_pages + page) * p.page_size + at
+        : (static_cast<int64_t>(b) * H + h) * a.seq + at;
+    *reinterpret_cast<uint32_t*>(cache + row * D + d) = packed;
+  }
+  // one thread per scale group writes the scale
+  if (groups == 1 ? threadIdx.x == 0 : d == 0) {
+    const int g = groups == 1 ? 0 : h;
+    if (stash_scale) store_from_f32(stash_scale, static_cast<int64_t>(b) * groups + g, a.scale_dtype, s);
+    if (write_cache && scale_out) {
+      const int64_t idx = paged
+          ? (static_cast<int64_t>(g) * p.total_pages + page) * p.page_size + at
+          : (static_cast<int64_t>(b) * groups + g) * a.seq + at;
+      store_from_f32(scale_out, idx, a.scale_dtype, s);
+    }
+  }
+}
+
 int32_t check_quant_common(int32_t heads, int32_t dim, int32_t in_dtype,
                            int32_t scale_dtype, int32_t scale_heads,
                            int32_t rounding) {
@@ -177,6 +266,19 @@ int32_t check_quant_common(int32_t heads, int32_t dim, int32_t in_dtype,
 int32_t launch_quant(const QuantParams& p, int32_t tokens, hipStream_t stream) {
   if (tokens == 0) return JPT_OK;
   dim3 grid(tokens, 2);
+  const jpt_quant_append_args& a = p.a;
+  const int d4 = a.dim / 4;
+  const bool vec = a.in_dtype == JPT_BF16 && a.heads * a.dim == 1024 && a.dim % 4 == 0 &&
+                   (a.scale_heads == 1 || (d4 <= 64 && (d4 & (d4 - 1)) == 0)) &&
+                   aligned(a.new_k, 8) && aligned(a.new_v, 8) && aligned(a.out_k, 4) && aligned(a.out_v, 4) &&
+                   aligned(a.cache_k, 4) && aligned(a.cache_v, 4);
+  if (vec) {
+    if (a.scale_dtype == JPT_BF16)
+      hipLaunchKernelGGL(quant_append_vec_kernel<true>, grid, dim3(256), 0, stream, p);
+    else
+      hipLaunchKernelGGL(quant_append_vec_kernel<false>, grid, dim3(256), 0, stream, p);
+    return launch_status("quant_append_vec_kernel");
+  }
   if (p.a.scale_dtype == JPT_BF16)
     hipLaunchKernelGGL(quant_append_kernel<true>, grid, dim3(256), 0, stream, p);
   else
