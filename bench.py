@@ -33,6 +33,11 @@ for _p in (ROOT, os.path.join(ROOT, "jetstream-pytorch_amd")):
 HBM_PEAK_GBPS = 8000.0
 B, HQ, HKV, D, S, LAYERS = 128, 32, 8, 128, 8192, 32
 SEED = 3
+PROBE_COPY_BYTES = 1 << 30
+# HBM bytes of one attention launch (decode kernel + merge kernel) on this
+# workload, from hardware counters (FETCH_SIZE + WRITE_SIZE, each calibrated on a
+# 1 GiB copy; see --probe-traffic).  A recorded measurement, not computed here.
+MEASURED_ATTN_TRAFFIC_BYTES = 163_210_000
 
 
 def seeded_lengths(torch):
@@ -147,6 +152,44 @@ def run_gpu(args):
               attn_bytes=attn_bytes(lengths), total_tokens=int(lengths.sum()))
 
 
+def run_traffic_probe(args):
+  """Work for a hardware-counter run (rocprofv3 --pmc FETCH_SIZE or WRITE_SIZE):
+  a few attention launches of the headline workload next to plain copies of a
+  buffer of known size, whose counter reading calibrates the counter's unit."""
+  import torch
+
+  from jetstream_pt_amd import attention_kernel as ak
+
+  dev = "cuda:0"
+  torch.cuda.set_device(0)
+  nl = 4
+  lengths = seeded_lengths(torch).to(dev)
+  k = torch.empty((nl, B, HKV, S, D), dtype=torch.int8, device=dev)
+  v = torch.empty_like(k)
+  for l in range(nl):
+    k[l].random_(-127, 128)
+    v[l].random_(-127, 128)
+  ks = torch.empty((nl, B, 1, S, 1), device=dev).uniform_(0.005, 0.05)
+  vs = torch.empty_like(ks).uniform_(0.005, 0.05)
+  g = torch.Generator(device=dev).manual_seed(SEED)
+  xq = torch.randn((B, HQ, 1, D), generator=g, device=dev).to(torch.bfloat16)
+  nk = torch.empty((B, HKV, 1, D), dtype=torch.int8, device=dev).random_(-127, 128)
+  nv = torch.empty_like(nk).random_(-127, 128)
+  nks = torch.empty((B, 1, 1, 1), device=dev).uniform_(0.005, 0.05)
+  nvs = torch.empty_like(nks).uniform_(0.005, 0.05)
+  plan, _ = ak.precompute_ragged_block_indices(lengths, B, HQ, HKV, S)
+  src = torch.empty(PROBE_COPY_BYTES // 4, dtype=torch.float32, device=dev).normal_()
+  dst = torch.empty_like(src)
+  for i in range(8):
+    ak.ragged_mha(xq, k, v, i % nl, None, plan.lengths, plan, None, ks, vs, new_key=nk, new_value=nv,
+                  new_k_scaler=nks, new_v_scaler=nvs)
+    dst.copy_(src)
+  torch.cuda.synchronize()
+  print(json.dumps({"probe": "traffic", "attention_launches": 8, "copies": 8,
+                    "copy_bytes_read": PROBE_COPY_BYTES, "copy_bytes_written": PROBE_COPY_BYTES,
+                    "attn_algorithmic_bytes": attn_bytes(lengths.cpu())}))
+
+
 def run_cpu_baseline(budget_s=20.0):
   """The oracle (CPU restatement of the reference path) on one layer of the
   same workload: Int8KVCacheGenerate.update + ragged_mha + new-token flash
@@ -196,10 +239,15 @@ def main():
   ap.add_argument("--layers", type=int, default=LAYERS)
   ap.add_argument("--no-cpu-baseline", action="store_true")
   ap.add_argument("--no-graph", action="store_true", help="launch every step from Python")
+  ap.add_argument("--probe-traffic", action="store_true",
+                  help="run a few attention launches and calibration copies for a counter run")
   args = ap.parse_args()
   if args.gpus != 1:
     sys.exit("bench.py measures one GPU: the path is built and measured on a single MI355X "
              "(--gpus must be 1)")
+  if args.probe_traffic:
+    run_traffic_probe(args)
+    return
   r = run_gpu(args)
   gbps = r["step_bytes"] / (r["ms_per_step"] * 1e-3) / 1e9
   attn_gbps = r["attn_bytes"] / (r["attn_ms"] * 1e-3) / 1e9
@@ -230,7 +278,8 @@ def main():
       "roofline": {
           "bound": "hbm", "kernel": "attn_decode_kernel<int8> + attn_merge_kernel (one attention launch)",
           "achieved": round(attn_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-          "frac": round(attn_gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+          "frac": round(attn_gbps / HBM_PEAK_GBPS, 4),
+          "traffic": MEASURED_ATTN_TRAFFIC_BYTES if args.layers == LAYERS else None,
           "us_per_launch": round(r["attn_ms"] * 1e3, 2), "algorithmic_bytes": r["attn_bytes"],
       },
   }
