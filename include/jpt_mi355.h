@@ -160,6 +160,41 @@ int32_t jpt_paged_append_quant_i8(const jpt_paged_quant_append_args* args,
                                   void* stream);
 
 /* ------------------------------------------------------------------------
+ * Prefill -> decode insert of one prompt into one slot, one layer.
+ *
+ * Replaces the cache part of Engine._insert_no_wrap (engine.py:371-488: a
+ * dynamic_update_slice of the prompt's K/V at position `start`, after
+ * quantize_tensor over (heads, dim) per token when the cache is int8) and of
+ * Engine._insert_wrap (:491-581: rows scattered to (start + t) mod seq).  With
+ * page_ids set it is the int8 counterpart of jpt_paged_insert for int8 pages
+ * (no reference counterpart): token t goes to page_ids[t / page_size], row
+ * t % page_size, and the rows of the last page past `tokens` are zero-filled.
+ *
+ * src_k/src_v (heads, tokens, dim) in in_dtype.  Dense: dst (batch, heads,
+ * seq, dim), scales (batch, scale_heads, seq).  Paged: dst (heads,
+ * total_pages, page_size, dim), scales (scale_heads, total_pages, page_size).
+ * dst_dtype == in_dtype copies; dst_dtype == JPT_I8 quantises with `rounding`
+ * (the reference inserts with JPT_ROUND_RNE, quantize.py:58-75), scales and
+ * intermediate results in scale_dtype as in jpt_kv_append_quant_i8.
+ * ---------------------------------------------------------------------- */
+typedef struct {
+  const void* src_k;
+  const void* src_v;
+  void* dst_k;
+  void* dst_v;
+  void* k_scale;
+  void* v_scale;
+  const int32_t* page_ids; /* device array of n_pages ids, or NULL (dense) */
+  int32_t n_pages;
+  int32_t tokens, heads, dim;
+  int32_t slot, batch, seq, start; /* dense */
+  int32_t total_pages, page_size;  /* paged */
+  int32_t in_dtype, dst_dtype, scale_dtype, scale_heads, rounding;
+} jpt_prefill_insert_args;
+
+int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void* stream);
+
+/* ------------------------------------------------------------------------
  * Decode attention.
  *
  * One argument block serves the three reference entry points:

@@ -1,0 +1,189 @@
+// Prefill -> decode insert: a prompt's K and V rows (heads, tokens, dim) written
+// into one slot of a dense cache (with ring wrap) or into the slot's pages,
+// either copied or quantised per token to int8 with the insert quantiser.
+//
+// One workgroup per (token, K|V).  HBM-bound data movement: reads the prompt
+// once (the quantising pass re-reads it from cache), writes codes and scales.
+#include "common.h"
+
+namespace jpt {
+namespace {
+
+struct InsertParams {
+  jpt_prefill_insert_args a;
+};
+
+template <bool ROUND_BF16>
+__device__ __forceinline__ float rnd(float x) {
+  return ROUND_BF16 ? round_to_bf16(x) : x;
+}
+
+// four consecutive elements of the source row as float
+__device__ __forceinline__ void load4(const void* src, int64_t i, int dtype, float* x) {
+  if (dtype == JPT_BF16) {
+    const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(src) + i);
+    x[0] = __uint_as_float(raw.x << 16);
+    x[1] = __uint_as_float(raw.x & 0xffff0000u);
+    x[2] = __uint_as_float(raw.y << 16);
+    x[3] = __uint_as_float(raw.y & 0xffff0000u);
+  } else {
+    const float4 raw = *reinterpret_cast<const float4*>(static_cast<const float*>(src) + i);
+    x[0] = raw.x; x[1] = raw.y; x[2] = raw.z; x[3] = raw.w;
+  }
+}
+
+// dim % 4 == 0.  The op order of the quantiser is that of
+// jpt_kv_append_quant_i8 (each op rounded to the scale dtype):
+//   trunc: a = absmax; s = a / 127;             q = x / s;      code = trunc(q)
+//   rne:   a = max(absmax, eps); s = a / 127; r = 1 / s; q = x * r;
+//          code = clamp(rint(q), -128, 127)
+template <bool BF16_MATH>
+__global__ void __launch_bounds__(256) prefill_insert_kernel(InsertParams p) {
+  const jpt_prefill_insert_args& a = p.a;
+  const int t = blockIdx.x;
+  const bool is_v = blockIdx.y == 1;
+  const void* src = is_v ? a.src_v : a.src_k;
+  char* dst = static_cast<char*>(is_v ? a.dst_v : a.dst_k);
+  void* scale_out = is_v ? a.v_scale : a.k_scale;
+  const bool paged = a.page_ids != nullptr;
+  const bool quant = a.dst_dtype == JPT_I8 && a.in_dtype != JPT_I8;
+  const int H = a.heads, D = a.dim, HD = H * D;
+  const int esz_in = a.in_dtype == JPT_F32 ? 4 : a.in_dtype == JPT_BF16 ? 2 : 1;
+  const int esz_out = quant ? 1 : esz_in;
+
+  // destination row of (this token, head h): element index row * D
+  int64_t pool_row = 0;  // dense: position in the slot's row; paged: row in the pool
+  if (paged) {
+    const int page = a.page_ids[t / a.page_size];
+    if (page < 0 || page >= a.total_pages) return;
+    pool_row = static_cast<int64_t>(page) * a.page_size + t % a.page_size;
+  } else {
+    int at = (a.start + t) % a.seq;
+    pool_row = at < 0 ? at + a.seq : at;
+  }
+  auto row_of = [&](int h) -> int64_t {
+    return paged ? static_cast<int64_t>(h) * a.total_pages * a.page_size + pool_row
+                 : (static_cast<int64_t>(a.slot) * H + h) * a.seq + pool_row;
+  };
+  auto scale_index = [&](int g) -> int64_t {
+    return paged ? static_cast<int64_t>(g) * a.total_pages * a.page_size + pool_row
+                 : (static_cast<int64_t>(a.slot) * a.scale_heads + g) * a.seq + pool_row;
+  };
+
+  if (t >= a.tokens) {  // paged only: the tail of the last page is zero-filled
+    for (int i = 4 * threadIdx.x; i < HD; i += 4 * blockDim.x) {
+      const int h = i / D, d = i - h * D;
+      char* out = dst + (row_of(h) * D + d) * esz_out;
+      if (esz_out == 1) *reinterpret_cast<uint32_t*>(out) = 0u;
+      else if (esz_out == 2) *reinterpret_cast<uint2*>(out) = make_uint2(0u, 0u);
+      else *reinterpret_cast<uint4*>(out) = make_uint4(0u, 0u, 0u, 0u);
+    }
+    return;
+  }
+  auto src_index = [&](int h, int d) -> int64_t { return (static_cast<int64_t>(h) * a.tokens + t) * D + d; };
+
+  if (!quant) {  // copy
+    for (int i = 4 * threadIdx.x; i < HD; i += 4 * blockDim.x) {
+      const int h = i / D, d = i - h * D;
+      const char* in = static_cast<const char*>(src) + src_index(h, d) * esz_in;
+      char* out = dst + (row_of(h) * D + d) * esz_in;
+      if (esz_in == 1) *reinterpret_cast<uint32_t*>(out) = *reinterpret_cast<const uint32_t*>(in);
+      else if (esz_in == 2) *reinterpret_cast<uint2*>(out) = *reinterpret_cast<const uint2*>(in);
+      else *reinterpret_cast<uint4*>(out) = *reinterpret_cast<const uint4*>(in);
+    }
+    return;
+  }
+
+  __shared__ float s_red[4];
+  __shared__ float s_scale[64];
+  const int groups = a.scale_heads;  // 1 or H
+  const int per_group = HD / groups;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int g = 0; g < groups; ++g) {
+    float m = 0.f;
+    for (int i = 4 * threadIdx.x; i < per_group; i += 4 * blockDim.x) {
+      const int e = g * per_group + i, h = e / D, d = e - h * D;
+      float x[4];
+      load4(src, src_index(h, d), a.in_dtype, x);
+      m = fmaxf(m, fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3]))));
+    }
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    if (lane == 0) s_red[wave] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float amax = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+      if (a.rounding == JPT_ROUND_RNE) amax = fmaxf(amax, rnd<BF16_MATH>(1e-5f));
+      s_scale[g] = rnd<BF16_MATH>(amax / 127.0f);
+    }
+    __syncthreads();
+  }
+  for (int i = 4 * threadIdx.x; i < HD; i += 4 * blockDim.x) {
+    const int h = i / D, d = i - h * D;
+    const float s = s_scale[groups == 1 ? 0 : h];
+    float x[4];
+    load4(src, src_index(h, d), a.in_dtype, x);
+    int code[4];
+    if (a.rounding == JPT_ROUND_TRUNC) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float q = rnd<BF16_MATH>(x[j] / s);
+        code[j] = (q != q) ? 0 : static_cast<int>(q);
+      }
+    } else {
+      const float r = rnd<BF16_MATH>(1.0f / s);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float q = rnd<BF16_MATH>(x[j] * r);
+        code[j] = static_cast<int>(fminf(fmaxf(rintf(q), -128.f), 127.f));
+      }
+    }
+    const uint32_t packed = (static_cast<uint32_t>(code[0]) & 0xffu) | ((static_cast<uint32_t>(code[1]) & 0xffu) << 8) |
+                            ((static_cast<uint32_t>(code[2]) & 0xffu) << 16) | (static_cast<uint32_t>(code[3]) << 24);
+    *reinterpret_cast<uint32_t*>(dst + row_of(h) * D + d) = packed;
+  }
+  if (threadIdx.x < groups) store_from_f32(scale_out, scale_index(threadIdx.x), a.scale_dtype, s_scale[threadIdx.x]);
+}
+
+}  // namespace
+}  // namespace jpt
+
+extern "C" int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void* stream) {
+  using namespace jpt;
+  JPT_REQUIRE(args != nullptr, "args is NULL");
+  const jpt_prefill_insert_args& a = *args;
+  JPT_REQUIRE(a.src_k && a.src_v && a.dst_k && a.dst_v, "NULL tensor argument");
+  JPT_REQUIRE(a.tokens >= 0 && a.heads > 0 && a.dim > 0, "tokens, heads, dim out of range");
+  JPT_REQUIRE(a.dim % 4 == 0, "dim must be a multiple of 4");
+  JPT_REQUIRE(a.in_dtype == JPT_BF16 || a.in_dtype == JPT_F32 || a.in_dtype == JPT_I8, "bad in_dtype");
+  const bool quant = a.dst_dtype == JPT_I8 && a.in_dtype != JPT_I8;
+  JPT_REQUIRE(quant || a.dst_dtype == a.in_dtype, "dst_dtype must be in_dtype (copy) or int8 (quantise)");
+  const int esz = a.in_dtype == JPT_F32 ? 4 : a.in_dtype == JPT_BF16 ? 2 : 1;
+  JPT_REQUIRE(aligned(a.src_k, 4 * esz) && aligned(a.src_v, 4 * esz), "source rows must be aligned to four elements");
+  const int esz_out = quant ? 1 : esz;
+  JPT_REQUIRE(aligned(a.dst_k, 4 * esz_out) && aligned(a.dst_v, 4 * esz_out), "destination must be aligned to four elements");
+  if (quant) {
+    JPT_REQUIRE(a.k_scale && a.v_scale, "k_scale/v_scale are NULL");
+    JPT_REQUIRE(a.scale_dtype == a.in_dtype || a.scale_dtype == JPT_F32, "scale_dtype must equal in_dtype or be f32");
+    JPT_REQUIRE(a.scale_heads == 1 || a.scale_heads == a.heads, "scale_heads must be 1 or heads");
+    JPT_REQUIRE(a.scale_heads <= 64, "per-head scales support at most 64 heads");
+    JPT_REQUIRE(a.scale_heads == 1 || a.dim % 4 == 0, "dim must be a multiple of 4");
+    JPT_REQUIRE(a.rounding == JPT_ROUND_TRUNC || a.rounding == JPT_ROUND_RNE, "bad rounding mode");
+  }
+  int32_t rows = a.tokens;
+  if (a.page_ids) {
+    JPT_REQUIRE(a.total_pages > 0 && a.page_size > 0 && a.n_pages >= 0, "paged geometry out of range");
+    JPT_REQUIRE(static_cast<int64_t>(a.n_pages) * a.page_size >= a.tokens, "too few pages for %d tokens", a.tokens);
+    rows = a.n_pages * a.page_size;
+  } else {
+    JPT_REQUIRE(a.seq > 0 && a.batch > 0 && a.slot >= 0 && a.slot < a.batch, "slot or seq out of range");
+    JPT_REQUIRE(a.tokens <= a.seq, "%d tokens do not fit a cache of %d positions", a.tokens, a.seq);
+  }
+  if (rows == 0) return JPT_OK;
+  InsertParams p{*args};
+  dim3 grid(rows, 2);
+  if (quant && a.scale_dtype == JPT_BF16)
+    hipLaunchKernelGGL(prefill_insert_kernel<true>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), p);
+  else
+    hipLaunchKernelGGL(prefill_insert_kernel<false>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), p);
+  return launch_status("prefill_insert_kernel");
+}

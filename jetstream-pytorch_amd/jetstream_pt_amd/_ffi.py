@@ -58,6 +58,17 @@ class PagedQuantAppendArgs(_c.Structure):
   ]
 
 
+class PrefillInsertArgs(_c.Structure):
+  _fields_ = [
+      ("src_k", _vp), ("src_v", _vp), ("dst_k", _vp), ("dst_v", _vp),
+      ("k_scale", _vp), ("v_scale", _vp), ("page_ids", _vp), ("n_pages", _i32),
+      ("tokens", _i32), ("heads", _i32), ("dim", _i32), ("slot", _i32),
+      ("batch", _i32), ("seq", _i32), ("start", _i32), ("total_pages", _i32),
+      ("page_size", _i32), ("in_dtype", _i32), ("dst_dtype", _i32),
+      ("scale_dtype", _i32), ("scale_heads", _i32), ("rounding", _i32),
+  ]
+
+
 class AttnArgs(_c.Structure):
   _fields_ = [
       ("q", _vp), ("k", _vp), ("v", _vp), ("k_scale", _vp), ("v_scale", _vp),
@@ -89,6 +100,7 @@ _sig("jpt_paged_insert", _i32, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, 
 _sig("jpt_paged_append", _i32, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_paged_gather", _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_paged_append_quant_i8", _i32, _c.POINTER(PagedQuantAppendArgs), _vp)
+_sig("jpt_prefill_insert", _i32, _c.POINTER(PrefillInsertArgs), _vp)
 _sig("jpt_attn_workspace_bytes", _i64, _c.POINTER(AttnArgs))
 _sig("jpt_attn_plan", _i32, _c.POINTER(AttnArgs), _i32, _vp)
 _sig("jpt_attn_ragged", _i32, _c.POINTER(AttnArgs), _vp)
@@ -108,7 +120,7 @@ _sig("jpt_pam_free_count", _i32, _vp, _i32p)
 EXPORTS = (
     "jpt_version", "jpt_last_error", "jpt_kv_scatter_lines",
     "jpt_kv_append_quant_i8", "jpt_paged_insert", "jpt_paged_append",
-    "jpt_paged_gather", "jpt_paged_append_quant_i8",
+    "jpt_paged_gather", "jpt_paged_append_quant_i8", "jpt_prefill_insert",
     "jpt_attn_workspace_bytes", "jpt_attn_plan", "jpt_attn_ragged", "jpt_attn_dense",
     "jpt_attn_paged", "jpt_lse_merge", "jpt_pam_create", "jpt_pam_destroy",
     "jpt_pam_tables", "jpt_pam_reserve_insert", "jpt_pam_reserve_decode",

@@ -1,0 +1,129 @@
+"""Prefill -> decode insert of one prompt into one batch slot.
+
+Mirrors the cache and bookkeeping part of the reference engine's insert
+(jetstream_pt/engine.py): `_insert_no_wrap` (:371-488), `_insert_wrap`
+(:491-581), `insert` (:606-626) and, for int8 pages, the paged insert
+(:583-604 with page_attention_manager.py:83-142).  Caches are updated in
+place by one kernel launch per layer (K and V together); with a quantised
+cache the prompt is quantised per token over (heads, dim) by the reference's
+insert quantiser (quantize.py:58-75: round half to even, clamp, eps 1e-5) in
+the prompt's dtype.
+"""
+
+import torch
+
+from . import _ffi
+
+
+def _rounding_code(rounding):
+  return {"trunc": _ffi.ROUND_TRUNC, "rne": _ffi.ROUND_RNE}[rounding]
+
+
+def _layer_views(cache, layer, n_layers):
+  """(k, v) of `layer`, given a stacked (L, B, H, S, D) pair or a list of
+  per-layer (k, v) pairs."""
+  if isinstance(cache, (list, tuple)) and isinstance(cache[0], (list, tuple)):
+    if len(cache) == 1 and cache[0][0].dim() == 5:  # reference: [(stacked_k, stacked_v)]
+      return cache[0][0][layer], cache[0][1][layer]
+    return cache[layer]
+  k, v = cache
+  return (k[layer], v[layer]) if k.dim() == 5 else (k, v)
+
+
+def insert_prefix_caches(prefix_caches, caches, cache_scales, slot, start, *, rounding="rne"):
+  """Writes the prompt's per-layer (key, value) pairs - each (1, heads, T, D) -
+  into slot `slot` of the decode caches at positions (start + t) mod S.
+
+  caches: list of per-layer (k, v) tensors (B, H, S, D), or [(k, v)] with
+  stacked (L, B, H, S, D) tensors (the reference's two DecodeState layouts).
+  cache_scales: None for float caches; else the scalers in the same layout,
+  each (B, Hs, S, 1) / (L, B, Hs, S, 1).  int8 caches are quantised into;
+  float caches take a copy (cast to the cache dtype first).
+  """
+  n_layers = len(prefix_caches)
+  for layer, (newk, newv) in enumerate(prefix_caches):
+    k, v = _layer_views(caches, layer, n_layers)
+    k, v = _ffi.dev(k, "cache_k"), _ffi.dev(v, "cache_v")
+    batch, heads, seq, dim = k.shape
+    if newk.dim() == 4:
+      newk, newv = newk[0], newv[0]
+    tokens = newk.shape[1]
+    quant = k.dtype == torch.int8 and newk.dtype != torch.int8
+    if not quant and newk.dtype != k.dtype:
+      newk, newv = newk.to(k.dtype), newv.to(v.dtype)
+    newk, newv = _ffi.dev(newk.contiguous(), "prefix key"), _ffi.dev(newv.contiguous(), "prefix value")
+    if newk.shape != (heads, tokens, dim):
+      raise ValueError(f"prefix key {tuple(newk.shape)} does not match cache {tuple(k.shape)}")
+    a = _ffi.PrefillInsertArgs(
+        src_k=_ffi.ptr(newk), src_v=_ffi.ptr(newv), dst_k=_ffi.ptr(k), dst_v=_ffi.ptr(v),
+        tokens=tokens, heads=heads, dim=dim, slot=int(slot), batch=batch, seq=seq,
+        start=int(start), in_dtype=_ffi.dtype_code(newk.dtype),
+        dst_dtype=_ffi.dtype_code(k.dtype))
+    if quant:
+      ks, vs = _layer_views(cache_scales, layer, n_layers)
+      ks, vs = _ffi.dev(ks, "k_scaler"), _ffi.dev(vs, "v_scaler")
+      a.k_scale, a.v_scale = _ffi.ptr(ks), _ffi.ptr(vs)
+      a.scale_dtype, a.scale_heads = _ffi.dtype_code(ks.dtype), ks.shape[1]
+      a.rounding = _rounding_code(rounding)
+    _ffi.check(_ffi.lib.jpt_prefill_insert(a, _ffi.stream()))
+
+
+def insert_prefix_pages_int8(prefix_caches, decode_caches, scale_pages, page_ids, *, rounding="rne"):
+  """int8 pages: per layer, quantises the prompt (1, heads, T, D) per token and
+  writes token t to page page_ids[t // ps], row t % ps; the rest of the last
+  page is zero-filled (as insert_prefill_cache does for float pages).
+  decode_caches / scale_pages: per-layer lists of (k, v) pairs."""
+  ids = _ffi.as_i32(page_ids, decode_caches[0][0].device)
+  for (newk, newv), (pk, pv), (ks, vs) in zip(prefix_caches, decode_caches, scale_pages):
+    pk, pv = _ffi.dev(pk, "pages_k"), _ffi.dev(pv, "pages_v")
+    heads, total, ps, dim = pk.shape
+    if newk.dim() == 4:
+      newk, newv = newk[0], newv[0]
+    newk, newv = _ffi.dev(newk.contiguous(), "prefix key"), _ffi.dev(newv.contiguous(), "prefix value")
+    a = _ffi.PrefillInsertArgs(
+        src_k=_ffi.ptr(newk), src_v=_ffi.ptr(newv), dst_k=_ffi.ptr(pk), dst_v=_ffi.ptr(pv),
+        k_scale=_ffi.ptr(_ffi.dev(ks, "k_scale_pages")), v_scale=_ffi.ptr(_ffi.dev(vs, "v_scale_pages")),
+        page_ids=_ffi.ptr(ids), n_pages=ids.numel(), tokens=newk.shape[1], heads=heads, dim=dim,
+        total_pages=total, page_size=ps, in_dtype=_ffi.dtype_code(newk.dtype), dst_dtype=_ffi.I8,
+        scale_dtype=_ffi.dtype_code(ks.dtype), scale_heads=ks.shape[0], rounding=_rounding_code(rounding))
+    _ffi.check(_ffi.lib.jpt_prefill_insert(a, _ffi.stream()))
+
+
+def insert(env, prefix_caches, prefix_seq_len, caches, cache_scales, slot, *, current_position=0,
+           mask=None, start=None, input_pos=None, lens=None):
+  """The reference's Engine.insert for dense caches: picks no-wrap or wrap as
+  engine.py:606-626 does, writes the caches (and scalers), and updates the
+  slot's row of the bookkeeping tensors that are given, in place:
+  mask (B, S) additive, start (B,), input_pos (B,), lens (B,).
+  Returns the first cache position written."""
+  seq = env.cache_sequence_length
+  padded = prefix_caches[0][0].shape[-2]
+  if env.ring_buffer:
+    start_insert = current_position - prefix_seq_len
+    end_insert = start_insert + padded
+    wrap = not (start_insert >= 0 and end_insert < seq)
+    cur = current_position
+  else:
+    wrap, cur = False, prefix_seq_len
+  if not wrap:
+    pos = cur - prefix_seq_len
+    insert_prefix_caches(prefix_caches, caches, cache_scales, slot, pos)
+    first = pos % seq
+    if mask is not None:
+      x = torch.arange(seq, device=mask.device)
+      mask[slot] = torch.where((x < cur) & (x >= pos), 0.0, float("-inf")).to(mask.dtype)
+  else:
+    first = (current_position - prefix_seq_len) % seq
+    insert_prefix_caches(prefix_caches, caches, cache_scales, slot, first)
+    if mask is not None:
+      x = torch.arange(seq, device=mask.device)
+      cond = ((x >= first) & (x < current_position)) if current_position > first else \
+          ((x >= first) | (x < current_position))
+      mask[slot] = torch.where(cond, 0.0, float("-inf")).to(mask.dtype)
+  if start is not None:
+    start[slot] = first
+  if input_pos is not None:
+    input_pos[slot] = prefix_seq_len
+  if lens is not None:
+    lens[slot] = 1
+  return first

@@ -28,6 +28,10 @@ class Env:
   paged_attention_total_num_pages: int = 0
   paged_attention_page_size: int = 64
 
+  @property
+  def cache_sequence_length(self):
+    return self.cache_len
+
   def __post_init__(self):
     requested = (
         self.lazy_cache_update,

@@ -1,0 +1,127 @@
+"""GPU parity: the prefill -> decode insert through the C ABI against the CPU
+oracle (engine.py:371-626 restated) on the same seeded inputs.  Cache bytes,
+codes, scales and bookkeeping are compared bit for bit."""
+
+import pytest
+import torch
+
+from oracle import Env as OEnv
+from oracle import insert as oins
+from oracle import quant as oquant
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def make_state(stacked, batch, heads, seq, dim, layers, quantized, scale_dtype=torch.bfloat16, seed=0):
+  g = torch.Generator().manual_seed(seed)
+  def cache():
+    if quantized:
+      return torch.randint(-127, 128, (batch, heads, seq, dim), generator=g, dtype=torch.int8)
+    return torch.randn((batch, heads, seq, dim), generator=g).to(torch.bfloat16)
+  def scale():
+    return torch.rand((batch, 1, seq, 1), generator=g).to(scale_dtype)
+  if stacked:
+    caches = [(torch.stack([cache() for _ in range(layers)]), torch.stack([cache() for _ in range(layers)]))]
+    scales = [(torch.stack([scale() for _ in range(layers)]), torch.stack([scale() for _ in range(layers)]))]
+  else:
+    caches = [(cache(), cache()) for _ in range(layers)]
+    scales = [(scale(), scale()) for _ in range(layers)]
+  return dict(caches=caches, cache_scales=scales if quantized else None,
+              mask=torch.zeros((batch, seq)), start=torch.zeros(batch, dtype=torch.int32),
+              input_pos=torch.zeros(batch, dtype=torch.int32), lens=torch.zeros(batch, dtype=torch.int32))
+
+
+def to_dev(state):
+  mv = lambda pairs: None if pairs is None else [(k.to(DEV), v.to(DEV)) for k, v in pairs]
+  return dict(caches=mv(state["caches"]), cache_scales=mv(state["cache_scales"]),
+              mask=state["mask"].to(DEV), start=state["start"].to(DEV),
+              input_pos=state["input_pos"].to(DEV), lens=state["lens"].to(DEV))
+
+
+def assert_same(dev_state, cpu_state):
+  for name in ("caches", "cache_scales"):
+    if cpu_state[name] is None:
+      continue
+    for (dk, dv), (ck, cv) in zip(dev_state[name], cpu_state[name]):
+      assert torch.equal(dk.cpu(), ck), name
+      assert torch.equal(dv.cpu(), cv), name
+  for name in ("mask", "start", "input_pos", "lens"):
+    assert torch.equal(dev_state[name].cpu(), cpu_state[name]), name
+
+
+def run_both(ring, quantized, shape, prompt, seq_len, slot, current_position=0, scale_dtype=torch.bfloat16,
+             prefix_dtype=torch.bfloat16):
+  from jetstream_pt_amd import insert as gins
+  from jetstream_pt_amd.environment import JetEngineEnvironment, JetEngineEnvironmentData
+  batch, heads, seq, dim, layers = shape
+  oenv = OEnv(batch_size=batch, num_layers=layers, cache_len=seq, ring_buffer=ring)
+  genv = JetEngineEnvironment(JetEngineEnvironmentData(
+      batch_size=batch, num_layers=layers, cache_sequence_length=seq, ring_buffer=ring))
+  cpu = make_state(oenv.generate_cache_stacked, batch, heads, seq, dim, layers, quantized, scale_dtype)
+  dev = to_dev(cpu)
+  g = torch.Generator().manual_seed(11)
+  mag = torch.logspace(-2, 1.5, prompt).reshape(1, 1, prompt, 1)
+  prefix = [((torch.randn((1, heads, prompt, dim), generator=g) * mag).to(prefix_dtype),
+             (torch.randn((1, heads, prompt, dim), generator=g) * mag).to(prefix_dtype)) for _ in range(layers)]
+  # the HIP quantiser works in the scalers' dtype (the prompt's dtype unless float32 scalers are used)
+  compute = torch.float32 if (quantized and scale_dtype == torch.float32) else None
+  oins.insert(oenv, prefix, seq_len, cpu, slot, current_position, compute_dtype=compute)
+  gins.insert(genv, [(k.to(DEV), v.to(DEV)) for k, v in prefix], seq_len, dev["caches"], dev["cache_scales"], slot,
+              current_position=current_position, mask=dev["mask"], start=dev["start"],
+              input_pos=dev["input_pos"], lens=dev["lens"])
+  torch.cuda.synchronize()
+  assert_same(dev, cpu)
+
+
+@pytest.mark.parametrize("quantized", [False, True])
+def test_left_aligned_stacked_insert(quantized):
+  run_both(False, quantized, (3, 2, 32, 8, 2), prompt=16, seq_len=11, slot=2)
+
+
+@pytest.mark.parametrize("quantized", [False, True])
+@pytest.mark.parametrize("current_position,seq_len,prompt", [(24, 10, 16), (3, 6, 8), (16, 8, 8), (31, 20, 24)])
+def test_ring_insert_wrap_and_no_wrap(quantized, current_position, seq_len, prompt):
+  run_both(True, quantized, (2, 2, 32, 8, 2), prompt=prompt, seq_len=seq_len, slot=1,
+           current_position=current_position)
+
+
+def test_llama3_shaped_quantised_insert_fp32_scales():
+  # 8 KV heads x 128, prompt padded to 1024, float32 scalers (the kernel's vector path)
+  run_both(False, True, (4, 8, 2048, 128, 2), prompt=1024, seq_len=1000, slot=3, scale_dtype=torch.float32)
+
+
+def test_float32_prefix_into_float32_quantiser():
+  run_both(False, True, (2, 4, 64, 16, 1), prompt=32, seq_len=30, slot=0, scale_dtype=torch.float32,
+           prefix_dtype=torch.float32)
+
+
+@pytest.mark.parametrize("tokens", [1, 64, 100, 130])
+def test_int8_paged_insert_equals_quantise_then_page_layout(tokens):
+  from jetstream_pt_amd import insert as gins
+  heads, total, ps, dim, layers = 4, 24, 64, 32, 2
+  n_pages = (tokens + ps - 1) // ps
+  g = torch.Generator().manual_seed(tokens)
+  page_ids = torch.randperm(total, generator=g)[:n_pages].to(torch.int32)
+  pools = [(torch.randint(-127, 128, (heads, total, ps, dim), generator=g, dtype=torch.int8),
+            torch.randint(-127, 128, (heads, total, ps, dim), generator=g, dtype=torch.int8)) for _ in range(layers)]
+  scale_pages = [(torch.rand((1, total, ps), generator=g), torch.rand((1, total, ps), generator=g)) for _ in range(layers)]
+  prefix = [((torch.randn((1, heads, tokens, dim), generator=g) * 2).to(torch.bfloat16),
+             torch.randn((1, heads, tokens, dim), generator=g).to(torch.bfloat16)) for _ in range(layers)]
+  dpools = [(k.to(DEV), v.to(DEV)) for k, v in pools]
+  dscales = [(k.to(DEV), v.to(DEV)) for k, v in scale_pages]
+  gins.insert_prefix_pages_int8([(k.to(DEV), v.to(DEV)) for k, v in prefix], dpools, dscales, page_ids)
+  torch.cuda.synchronize()
+  for layer in range(layers):
+    for which in (0, 1):
+      codes, scales = oquant.quantize_insert(prefix[layer][which].float())  # float32 scales: quantiser in float32
+      want = pools[layer][which].clone()
+      want_s = scale_pages[layer][which].clone()
+      padded = torch.zeros((heads, n_pages * ps, dim), dtype=torch.int8)
+      padded[:, :tokens, :] = codes[0]
+      want[:, page_ids.long(), :, :] = padded.reshape(heads, n_pages, ps, dim)
+      flat = want_s[0, page_ids.long(), :].reshape(-1)
+      flat[:tokens] = scales.reshape(-1)
+      want_s[0, page_ids.long(), :] = flat.reshape(n_pages, ps)
+      assert torch.equal(dpools[layer][which].cpu(), want)
+      assert torch.equal(dscales[layer][which].cpu(), want_s)
