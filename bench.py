@@ -1,9 +1,9 @@
 """Benchmark of the decode-time KV-cache hot path on one MI355X.
 
-Workload (BASELINE.json configs[2], the headline): ragged GQA decode
-attention for one Llama-3-8B layer - batch 128, 32 q heads / 8 KV heads,
-head_dim 128, cache length 8192, int8 KV codes with fp32 per-token scales,
-per-slot lengths log-normal (median 400, sigma 1) clipped to [16, 8192].
+Headline workload (BASELINE.json configs[2], `--workload c3`, the default):
+ragged GQA decode attention for one Llama-3-8B layer - batch 128, 32 q heads /
+8 KV heads, head_dim 128, cache length 8192, int8 KV codes with fp32 per-token
+scales, per-slot lengths log-normal (median 400, sigma 1) clipped to [16, 8192].
 
 A step is one layer-step of the production left-aligned mode: fused int8
 quantise + stash of the new token, then ragged attention over the cache with
@@ -13,9 +13,19 @@ a stacked cache (64 GiB of codes), so every step streams cold data; once per
 stashed tokens into the cache (both inside the timed region).
 
 Prints one JSON line.  `value` is algorithmic bytes of the layer-step divided
-by its time; `roofline` is the attention kernel alone (a separate timed loop
+by its time; `roofline` is the attention launch alone (a separate timed loop
 of attention launches only); `cpu_baseline` times the CPU oracle's
 restatement of the reference path on the host cores.
+
+The other configurations of BASELINE.json are parity-test cases; `--workload
+c1|c2|c4|c5` times them the same way for the record (same JSON shape, no
+cpu_baseline):
+  c1  dense bf16 eager update + dense attention, B=8, 32 heads, S=1024
+  c2  int8 MHA decode step, B=96, 32 heads, S=2048, lengths U[128, 2048]
+  c4  paged bf16, B=256, 64 q / 8 kv heads, 32768 pages of 64, host page
+      allocation every decode step, paged append + paged attention
+  c5  paged int8, 32 layers, B=256, 32 q / 8 kv heads, 16384 pages of 64 per
+      layer; every decode step frees 16 slots and inserts 16 new prompts
 """
 
 import argparse
@@ -31,92 +41,315 @@ for _p in (ROOT, os.path.join(ROOT, "jetstream-pytorch_amd")):
     sys.path.insert(0, _p)
 
 HBM_PEAK_GBPS = 8000.0
-B, HQ, HKV, D, S, LAYERS = 128, 32, 8, 128, 8192, 32
+D = 128
+B, HQ, HKV, S, LAYERS = 128, 32, 8, 8192, 32  # the headline workload
 SEED = 3
 PROBE_COPY_BYTES = 1 << 30
-# HBM bytes of one attention launch (decode kernel + merge kernel) on this
-# workload, from hardware counters (FETCH_SIZE + WRITE_SIZE, each calibrated on a
-# 1 GiB copy; see --probe-traffic).  A recorded measurement, not computed here.
+# HBM bytes of one attention launch (decode kernel + merge kernel) on the
+# headline workload, from hardware counters (FETCH_SIZE + WRITE_SIZE, each
+# calibrated on a 1 GiB copy; see --probe-traffic).  A recorded measurement,
+# not computed here.
 MEASURED_ATTN_TRAFFIC_BYTES = 163_210_000
+DEV = "cuda:0"
 
 
-def seeded_lengths(torch):
-  g = torch.Generator().manual_seed(SEED)
-  z = torch.randn(B, generator=g, dtype=torch.float64)
-  return torch.clamp(torch.round(torch.exp(math.log(400.0) + z)), 16, S).to(torch.int32)
+def seeded_lengths(torch, batch=B, median=400.0, lo=16, hi=S, seed=SEED):
+  g = torch.Generator().manual_seed(seed)
+  z = torch.randn(batch, generator=g, dtype=torch.float64)
+  return torch.clamp(torch.round(torch.exp(math.log(median) + z)), lo, hi).to(torch.int32)
+
+
+def uniform_lengths(torch, batch, lo, hi, seed):
+  g = torch.Generator().manual_seed(seed)
+  return torch.randint(lo, hi + 1, (batch,), generator=g, dtype=torch.int32)
+
+
+def dense_attn_bytes(total, batch, hq, hkv, e_kv, scales, new_token, e_scale=4):
+  """Algorithmic bytes of one attention launch over `total` attended
+  positions: K and V of those positions, their per-token scales (shared by all
+  heads), q in and o out (bf16), the lengths, and the new token if fused."""
+  kv = total * hkv * D * 2 * e_kv
+  sc = total * e_scale * 2 if scales else 0
+  qo = batch * hq * D * 2 * 2
+  new = (batch * hkv * D * 2 * e_kv + (batch * e_scale * 2 if scales else 0)) if new_token else 0
+  return kv + sc + qo + new + batch * 4
 
 
 def attn_bytes(lengths):
-  """Algorithmic bytes of one attention launch: int8 K and V codes of the
-  attended positions, their fp32 scales (one per token, shared by all heads),
-  q in and o out (bf16), the lengths, and the new token's codes and scales."""
-  total = int(lengths.sum())
-  kv = total * HKV * D * 2
-  scales = total * 4 * 2
-  qo = B * HQ * D * 2 * 2
-  new_tok = B * HKV * D * 2 + B * 4 * 2
-  return kv + scales + qo + new_tok + B * 4
+  """The headline workload's attention launch."""
+  return dense_attn_bytes(int(lengths.sum()), B, HQ, HKV, 1, True, True)
 
 
-def append_bytes():
-  """Quantise + stash: bf16 K and V in, int8 codes and fp32 scales out."""
-  return B * HKV * D * (2 + 1) * 2 + B * 4 * 2
+# ---- workloads -------------------------------------------------------------------
+# A builder returns a dict: step(i) and attn_only(i) enqueue layer-step i;
+# step_bytes / attn_bytes are algorithmic bytes per layer-step / attention launch;
+# graph says whether a pass over the layers may be captured in a HIP graph.
 
 
-def finalize_bytes_per_layer():
-  """finalize(): per layer, codes and scales read from the stash and written
-  into the cache."""
-  return (B * HKV * D + B * 4) * 2 * 2
-
-
-def run_gpu(args):
-  import torch
-
+def build_dense_int8(torch, nl, batch, hq, hkv, seq, lengths, name):
+  """Left-aligned production mode (lazy update, stacked int8 cache, ragged
+  attention with the new token fused): the shape of c2 and c3."""
   from jetstream_pt_amd import attention_kernel as ak
   from jetstream_pt_amd import cache_manager as cm
   from jetstream_pt_amd import layers
   from jetstream_pt_amd.environment import JetEngineEnvironment, JetEngineEnvironmentData
 
-  dev = "cuda:0"
-  torch.cuda.set_device(0)
-  lengths = seeded_lengths(torch)
-  nl = args.layers
-  env = JetEngineEnvironment(JetEngineEnvironmentData(batch_size=B, num_layers=nl, ring_buffer=False))
-  shape = (nl, B, HKV, S, D)
-  cache = cm.Int8KVCacheGenerate.empty(shape, dev, env, scale_heads=1, scale_dtype=torch.float32)
+  env = JetEngineEnvironment(JetEngineEnvironmentData(batch_size=batch, num_layers=nl, ring_buffer=False))
+  cache = cm.Int8KVCacheGenerate.empty((nl, batch, hkv, seq, D), DEV, env, scale_heads=1,
+                                       scale_dtype=torch.float32)
   for l in range(nl):  # codes uniform [-127, 127], scales U(0.005, 0.05)
     cache.cache_k[l].random_(-127, 128)
     cache.cache_v[l].random_(-127, 128)
     cache.k_scaler[l].uniform_(0.005, 0.05)
     cache.v_scaler[l].uniform_(0.005, 0.05)
-  g = torch.Generator(device=dev).manual_seed(SEED)
-  xq = torch.randn((B, HQ, 1, D), generator=g, device=dev).to(torch.bfloat16)
-  xk = torch.randn((B, HKV, 1, D), generator=g, device=dev).to(torch.bfloat16)
-  xv = torch.randn((B, HKV, 1, D), generator=g, device=dev).to(torch.bfloat16)
-  pos = lengths.to(dev)
+  g = torch.Generator(device=DEV).manual_seed(SEED)
+  xq = torch.randn((batch, hq, 1, D), generator=g, device=DEV).to(torch.bfloat16)
+  xk = torch.randn((batch, hkv, 1, D), generator=g, device=DEV).to(torch.bfloat16)
+  xv = torch.randn((batch, hkv, 1, D), generator=g, device=DEV).to(torch.bfloat16)
+  pos = lengths.to(DEV)
   cache.input_pos = pos
   kernels = [layers.Int8KVAttentionKernel(env, l) for l in range(nl)]
   state = {"plan": None}
 
-  def layer_step(i):
+  def step(i):
     l = i % nl
     if l == 0:
-      state["plan"], _ = ak.precompute_ragged_block_indices(pos, B, HQ, HKV, S)
+      state["plan"], _ = ak.precompute_ragged_block_indices(pos, batch, hq, hkv, seq)
     plan = state["plan"]
     out = kernels[l](xq, xk, xv, None, cache, start=None, end=plan.lengths, ragged_batch_index=plan)
     if l == nl - 1:
       cache.finalize()
     return out
 
+  plan, _ = ak.precompute_ragged_block_indices(pos, batch, hq, hkv, seq)
+  new = dict(new_key=cache.new_ks[0], new_value=cache.new_vs[0],
+             new_k_scaler=cache.new_k_scaler[0], new_v_scaler=cache.new_v_scaler[0])
+
+  def attn_only(i):
+    return ak.ragged_mha(xq, cache.cache_k, cache.cache_v, i % nl, None, plan.lengths, plan, None,
+                         cache.k_scaler, cache.v_scaler, **new)
+
+  total = int(lengths.sum())
+  ab = dense_attn_bytes(total, batch, hq, hkv, 1, True, True)
+  append = batch * hkv * D * (2 + 1) * 2 + batch * 4 * 2           # bf16 in, codes + fp32 scales out
+  finalize = (batch * hkv * D + batch * 4) * 2 * 2                # per layer: stash read, cache written
+  return dict(step=step, attn_only=attn_only, step_bytes=ab + append + finalize, attn_bytes=ab, graph=True,
+              cache=cache, lengths=lengths, xq=xq, xk=xk, xv=xv, env=env,
+              config={"workload": name, "batch": batch, "q_heads": hq, "kv_heads": hkv, "head_dim": D,
+                      "max_cache_len": seq, "layers_rotated": nl, "cached_tokens": total,
+                      "kv": "int8 codes + fp32 per-token scales"},
+              kernel="attn_decode_kernel<int8> + attn_merge_kernel (one attention launch)")
+
+
+def build_c3(torch, args):
+  lengths = seeded_lengths(torch)
+  w = build_dense_int8(torch, args.layers or LAYERS, B, HQ, HKV, S, lengths,
+                       "C3 ragged GQA int8 decode layer-step: KV quantise+stash, ragged attention with "
+                       "fused new token, finalize amortised over the layers")
+  w["config"]["lengths"] = "log-normal(median 400, sigma 1) in [16, 8192], seed 3"
+  return w
+
+
+def build_c2(torch, args):
+  lengths = uniform_lengths(torch, 96, 128, 2047, seed=2)
+  w = build_dense_int8(torch, args.layers or 32, 96, 32, 32, 2048, lengths,
+                       "C2 int8 MHA decode layer-step: KV quantise+stash, ragged attention with fused new "
+                       "token, finalize amortised over the layers")
+  w["config"]["lengths"] = "uniform [128, 2047], seed 2"
+  return w
+
+
+def build_c1(torch, args):
+  """Dense bf16 eager per-slot update + dense attention over the whole cache
+  with an additive mask."""
+  from jetstream_pt_amd import attention_kernel as ak
+  from jetstream_pt_amd import cache_manager as cm
+  from jetstream_pt_amd import layers
+  from jetstream_pt_amd.environment import JetEngineEnvironment, JetEngineEnvironmentData
+
+  nl, batch, heads, seq = args.layers or 32, 8, 32, 1024
+  env = JetEngineEnvironment(JetEngineEnvironmentData(
+      batch_size=batch, num_layers=nl, cache_sequence_length=seq, testing=True, ring_buffer=False,
+      lazy_cache_update=False, ragged_mha=False, flash_attention=False, generate_cache_stacked=False,
+      new_cache_stacked=False))
+  g = torch.Generator().manual_seed(1)
+  pos = torch.randint(0, seq, (batch,), generator=g, dtype=torch.int32)
+  gd = torch.Generator(device=DEV).manual_seed(1)
+  caches = []
+  x = torch.arange(seq).reshape(1, 1, seq, 1)
+  live = (x < pos.reshape(batch, 1, 1, 1)).to(DEV)
+  for _ in range(nl):
+    k = torch.randn((batch, heads, seq, D), generator=gd, device=DEV).to(torch.bfloat16) * live
+    v = torch.randn((batch, heads, seq, D), generator=gd, device=DEV).to(torch.bfloat16) * live
+    caches.append(cm.KVCacheGenerate(k, v, pos.to(DEV), None, env=env))
+  xq = torch.randn((batch, heads, 1, D), generator=gd, device=DEV).to(torch.bfloat16)
+  xk = torch.randn((batch, heads, 1, D), generator=gd, device=DEV).to(torch.bfloat16)
+  xv = torch.randn((batch, heads, 1, D), generator=gd, device=DEV).to(torch.bfloat16)
+  mask = torch.where(torch.arange(seq).reshape(1, 1, 1, seq) <= pos.reshape(batch, 1, 1, 1), 0.0,
+                     float("-inf")).to(DEV)
+  kernels = [layers.AttentionKernel(env, l) for l in range(nl)]
+
+  def step(i):
+    l = i % nl
+    return kernels[l](xq, xk, xv, mask, caches[l])
+
+  def attn_only(i):
+    c = caches[i % nl]
+    return ak.dense_attention(xq, c.cache_k, c.cache_v, mask=mask)
+
+  ab = batch * heads * seq * D * 2 * 2 + batch * seq * 4 + batch * heads * D * 2 * 2
+  append = batch * heads * D * 2 * 2 * 2
+  return dict(step=step, attn_only=attn_only, step_bytes=ab + append, attn_bytes=ab, graph=True,
+              caches=caches, pos=pos, mask=mask, xq=xq, xk=xk, xv=xv, env=env,
+              config={"workload": "C1 dense bf16 eager layer-step: per-slot KV line write, dense attention over "
+                                  "all 1024 positions with an additive mask",
+                      "batch": batch, "q_heads": heads, "kv_heads": heads, "head_dim": D,
+                      "max_cache_len": seq, "layers_rotated": nl, "kv": "bf16"},
+              kernel="attn_decode_kernel<bf16, mask> + attn_merge_kernel (one attention launch)")
+
+
+def build_paged(torch, args, int8):
+  """c4 (bf16 pages) / c5 (int8 pages, prompt churn): host page allocation once
+  per decode step, then per layer a paged append and a paged attention."""
+  import numpy as np
+
+  from jetstream_pt_amd import attention_kernel as ak
+  from jetstream_pt_amd import cache_manager as cm
+  from jetstream_pt_amd import insert as gins
+  from jetstream_pt_amd import layers
+  from jetstream_pt_amd.environment import JetEngineEnvironment, JetEngineEnvironmentData
+  from jetstream_pt_amd.page_attention_manager import PageAttentionManager
+
+  if int8:
+    nl, batch, hq, hkv, ps, total, max_pages, seed = args.layers or 32, 256, 32, 8, 64, 16384, 64, 5
+    lengths = seeded_lengths(torch, batch, 600.0, 16, 4096 - 256, seed).numpy().astype(np.int32)
+  else:
+    nl, batch, hq, hkv, ps, total, max_pages, seed = args.layers or 4, 256, 64, 8, 64, 32768, 128, 4
+    lengths = uniform_lengths(torch, batch, 32, 2048, seed).numpy().astype(np.int32)
+  env = JetEngineEnvironment(JetEngineEnvironmentData(
+      batch_size=batch, num_layers=nl, paged_attention_total_num_pages=total, paged_attention_page_size=ps))
+  rng = np.random.default_rng(seed)
+  pam = PageAttentionManager(batch, total, ps, max_pages, free_list_order=rng.permutation(total).astype(np.int32))
+  for slot in range(batch):
+    pam.reserve_pages_insert(slot, int(lengths[slot]))
+  e_kv = 1 if int8 else 2
+  kdt = torch.int8 if int8 else torch.bfloat16
+  pools_k = torch.empty((nl, hkv, total, ps, D), dtype=kdt, device=DEV)
+  pools_v = torch.empty_like(pools_k)
+  for l in range(nl):
+    if int8:
+      pools_k[l].random_(-127, 128)
+      pools_v[l].random_(-127, 128)
+    else:
+      pools_k[l].normal_()
+      pools_v[l].normal_()
+  sk = sv = None
+  if int8:
+    sk = torch.empty((nl, 1, total, ps), device=DEV).uniform_(0.005, 0.05)
+    sv = torch.empty((nl, 1, total, ps), device=DEV).uniform_(0.005, 0.05)
+  gd = torch.Generator(device=DEV).manual_seed(seed)
+  xq = torch.randn((batch, hq, 1, D), generator=gd, device=DEV).to(torch.bfloat16)
+  xk = torch.randn((batch, hkv, 1, D), generator=gd, device=DEV).to(torch.bfloat16)
+  xv = torch.randn((batch, hkv, 1, D), generator=gd, device=DEV).to(torch.bfloat16)
+  prompt_k = prompt_v = None
+  if int8:
+    caches = [cm.Int8PageKVCacheGenerate(pools_k[l], pools_v[l], sk[l], sv[l], pam, None, env=env) for l in range(nl)]
+    kernels = [layers.Int8KVAttentionKernel(env, l) for l in range(nl)]
+    prompt_k = torch.randn((nl, hkv, 1024, D), generator=gd, device=DEV).to(torch.bfloat16)
+    prompt_v = torch.randn((nl, hkv, 1024, D), generator=gd, device=DEV).to(torch.bfloat16)
+  else:
+    caches = [cm.PageKVCacheGenerate(pools_k[l], pools_v[l], pam, None, env=env) for l in range(nl)]
+    kernels = [layers.AttentionKernel(env, l) for l in range(nl)]
+  state = {"lens": lengths.copy(), "decode_steps": 0, "attended": 0, "pages": 0, "inserted": 0, "log": []}
+  churn = 16 if int8 else 0
+
+  def host_step():
+    """What the engine does on the host once per decode step."""
+    lens = state["lens"]
+    if churn:
+      for slot in rng.choice(batch, churn, replace=False):
+        pam.free_pages_resource(int(slot))
+        n = int(rng.integers(64, 1025))
+        _, ids = pam.reserve_pages_insert(int(slot), n)
+        ids = np.array(ids, dtype=np.int32)
+        gins.insert_prefix_pages_int8_stacked(prompt_k[:, :, :n], prompt_v[:, :, :n], pools_k, pools_v, sk, sv, ids)
+        lens[slot] = n
+        state["inserted"] += n
+        state["log"].append(("insert", int(slot), n, ids))
+    pam.fill_new_pages(lens)
+    idx_host = pam.get_page_token_indices(lens)
+    idx = torch.from_numpy(idx_host).to(DEV)
+    state["log"].append(("decode", lens.copy(), idx_host))
+    lens += 1
+    for c in caches:
+      c.page_token_indices = idx
+    state["decode_steps"] += 1
+    state["attended"] += int(lens.sum())
+    state["pages"] += int(((lens + ps - 1) // ps).sum())
+
+  def step(i):
+    l = i % nl
+    if l == 0:
+      host_step()
+    return kernels[l](xq, xk, xv, None, caches[l])
+
+  def attn_only(i):
+    l = i % nl
+    lens_d, table = pam.device_tables(DEV)
+    return ak.call_paged_attention(env, xq.squeeze(2), pools_k[l], pools_v[l], lens_d, table,
+                                   k_scaler=sk[l] if int8 else None, v_scaler=sv[l] if int8 else None)
+
+  def bytes_now():
+    """Average algorithmic bytes per layer-step / attention launch over the
+    decode steps run so far (lengths grow by one per step)."""
+    n = max(state["decode_steps"], 1)
+    att, pages = state["attended"] / n, state["pages"] / n
+    ab = att * hkv * D * 2 * e_kv + (att * 4 * 2 if int8 else 0) + batch * hq * D * 2 * 2 + pages * 4 + batch * 4
+    append = batch * hkv * D * (2 * 2 + 2 * e_kv) + (batch * 4 * 2 if int8 else 0)
+    ins = state["inserted"] / n * (hkv * D * 2 * (2 + 1) + 4 * 2) if int8 else 0   # per layer
+    return ab + append + ins, ab
+
+  name = ("C5 paged int8 layer-step: per decode step 16 slots freed and 16 prompts quantised into pages (all "
+          "layers), host page allocation; per layer quantised paged append + paged attention" if int8 else
+          "C4 paged bf16 layer-step: host page allocation per decode step; per layer paged append + paged attention")
+  return dict(step=step, attn_only=attn_only, bytes_now=bytes_now, graph=False, pam=pam, pools=(pools_k, pools_v),
+              scale_pages=(sk, sv), caches=caches, state=state, xq=xq, xk=xk, xv=xv, env=env,
+              prompts=(prompt_k, prompt_v), initial_lengths=lengths,
+              config={"workload": name, "batch": batch, "q_heads": hq, "kv_heads": hkv, "head_dim": D,
+                      "page_size": ps, "total_pages": total, "max_pages_per_seq": max_pages, "layers_rotated": nl,
+                      "kv": "int8 pages + fp32 scale pages" if int8 else "bf16 pages"},
+              kernel=("attn_decode_kernel<int8, paged>" if int8 else "attn_decode_kernel<bf16, paged>") +
+                     " + attn_merge_kernel (one attention launch)")
+
+
+def build_c4(torch, args):
+  return build_paged(torch, args, False)
+
+
+def build_c5(torch, args):
+  return build_paged(torch, args, True)
+
+
+WORKLOADS = {"c1": build_c1, "c2": build_c2, "c3": build_c3, "c4": build_c4, "c5": build_c5}
+
+
+def run_gpu(args):
+  import torch
+
+  torch.cuda.set_device(0)
+  w = WORKLOADS[args.workload](torch, args)
+  nl = w["config"]["layers_rotated"]
+  use_graph = w["graph"] and not args.no_graph
+
   def timed(fn, steps, warmup):
     """fn(i) enqueues step i.  Whole passes over the layers are replayed from
-    one captured HIP graph (what a serving loop does with a launch-bound
-    decode step); a remainder of steps runs eagerly."""
+    one captured HIP graph where the workload allows (what a serving loop does
+    with a launch-bound decode step); a remainder of steps runs eagerly."""
     for i in range(max(warmup, nl)):
       fn(i)
     torch.cuda.synchronize()
     graph = None
-    if not args.no_graph and steps >= nl:
+    if use_graph and steps >= nl:
       graph = torch.cuda.CUDAGraph()
       with torch.cuda.graph(graph):
         for i in range(nl):
@@ -136,20 +369,13 @@ def run_gpu(args):
     torch.cuda.synchronize()
     return start.elapsed_time(stop) / steps
 
-  ms_per_step = timed(layer_step, args.steps, args.warmup)
-
-  # one attention launch alone (decode kernel + partial-merge kernel), same inputs
-  plan, _ = ak.precompute_ragged_block_indices(pos, B, HQ, HKV, S)
-  new = dict(new_key=cache.new_ks[0], new_value=cache.new_vs[0],
-             new_k_scaler=cache.new_k_scaler[0], new_v_scaler=cache.new_v_scaler[0])
-  def attn_only(i):
-    return ak.ragged_mha(xq, cache.cache_k, cache.cache_v, i % nl, None, plan.lengths, plan, None,
-                         cache.k_scaler, cache.v_scaler, **new)
-  attn_ms = timed(attn_only, args.steps, args.warmup)
-
-  step_bytes = attn_bytes(lengths) + append_bytes() + finalize_bytes_per_layer()
-  return dict(ms_per_step=ms_per_step, attn_ms=attn_ms, step_bytes=step_bytes,
-              attn_bytes=attn_bytes(lengths), total_tokens=int(lengths.sum()))
+  ms_per_step = timed(w["step"], args.steps, args.warmup)
+  if "bytes_now" in w:
+    w["step_bytes"], w["attn_bytes"] = w["bytes_now"]()
+  attn_ms = timed(w["attn_only"], args.steps, args.warmup)
+  w.update(ms_per_step=ms_per_step, attn_ms=attn_ms, launch="hip graph of one pass over the layers" if use_graph
+           else "python")
+  return w
 
 
 def run_traffic_probe(args):
@@ -160,25 +386,24 @@ def run_traffic_probe(args):
 
   from jetstream_pt_amd import attention_kernel as ak
 
-  dev = "cuda:0"
   torch.cuda.set_device(0)
   nl = 4
-  lengths = seeded_lengths(torch).to(dev)
-  k = torch.empty((nl, B, HKV, S, D), dtype=torch.int8, device=dev)
+  lengths = seeded_lengths(torch).to(DEV)
+  k = torch.empty((nl, B, HKV, S, D), dtype=torch.int8, device=DEV)
   v = torch.empty_like(k)
   for l in range(nl):
     k[l].random_(-127, 128)
     v[l].random_(-127, 128)
-  ks = torch.empty((nl, B, 1, S, 1), device=dev).uniform_(0.005, 0.05)
+  ks = torch.empty((nl, B, 1, S, 1), device=DEV).uniform_(0.005, 0.05)
   vs = torch.empty_like(ks).uniform_(0.005, 0.05)
-  g = torch.Generator(device=dev).manual_seed(SEED)
-  xq = torch.randn((B, HQ, 1, D), generator=g, device=dev).to(torch.bfloat16)
-  nk = torch.empty((B, HKV, 1, D), dtype=torch.int8, device=dev).random_(-127, 128)
+  g = torch.Generator(device=DEV).manual_seed(SEED)
+  xq = torch.randn((B, HQ, 1, D), generator=g, device=DEV).to(torch.bfloat16)
+  nk = torch.empty((B, HKV, 1, D), dtype=torch.int8, device=DEV).random_(-127, 128)
   nv = torch.empty_like(nk).random_(-127, 128)
-  nks = torch.empty((B, 1, 1, 1), device=dev).uniform_(0.005, 0.05)
+  nks = torch.empty((B, 1, 1, 1), device=DEV).uniform_(0.005, 0.05)
   nvs = torch.empty_like(nks).uniform_(0.005, 0.05)
   plan, _ = ak.precompute_ragged_block_indices(lengths, B, HQ, HKV, S)
-  src = torch.empty(PROBE_COPY_BYTES // 4, dtype=torch.float32, device=dev).normal_()
+  src = torch.empty(PROBE_COPY_BYTES // 4, dtype=torch.float32, device=DEV).normal_()
   dst = torch.empty_like(src)
   for i in range(8):
     ak.ragged_mha(xq, k, v, i % nl, None, plan.lengths, plan, None, ks, vs, new_key=nk, new_value=nv,
@@ -192,7 +417,7 @@ def run_traffic_probe(args):
 
 def run_cpu_baseline(budget_s=20.0):
   """The oracle (CPU restatement of the reference path) on one layer of the
-  same workload: Int8KVCacheGenerate.update + ragged_mha + new-token flash
+  headline workload: Int8KVCacheGenerate.update + ragged_mha + new-token flash
   attention + merge, on the host cores."""
   import torch
 
@@ -225,7 +450,7 @@ def run_cpu_baseline(budget_s=20.0):
     times.append(time.perf_counter() - t0)
   times.sort()
   med = times[len(times) // 2]
-  nbytes = attn_bytes(lengths) + append_bytes()
+  nbytes = attn_bytes(lengths) + B * HKV * D * (2 + 1) * 2 + B * 4 * 2
   return dict(value=round(nbytes / med / 1e9, 3), unit="GB/s", cores=cores, kind="port",
               sample=f"one full layer-step (all {B} slots, {int(lengths.sum())} cached tokens), "
                      f"median of {len(times)} runs, {med * 1e3:.1f} ms each")
@@ -236,7 +461,8 @@ def main():
   ap.add_argument("--gpus", type=int, default=1)
   ap.add_argument("--steps", type=int, default=640)
   ap.add_argument("--warmup", type=int, default=64)
-  ap.add_argument("--layers", type=int, default=LAYERS)
+  ap.add_argument("--layers", type=int, default=0, help="cache layers to rotate over (0 = the workload's own)")
+  ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c3")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   ap.add_argument("--no-graph", action="store_true", help="launch every step from Python")
   ap.add_argument("--probe-traffic", action="store_true",
@@ -251,6 +477,10 @@ def main():
   r = run_gpu(args)
   gbps = r["step_bytes"] / (r["ms_per_step"] * 1e-3) / 1e9
   attn_gbps = r["attn_bytes"] / (r["attn_ms"] * 1e-3) / 1e9
+  headline = args.workload == "c3"
+  cfg = dict(r["config"])
+  cfg["launch"] = r["launch"]
+  model_layers = cfg["layers_rotated"] if args.workload == "c5" else LAYERS
   line = {
       "metric": "decode-attn HBM GB/s (% of 8 TB/s) + us/layer, Llama-3-8B GQA int8 B=128",
       "value": round(gbps, 1),
@@ -264,26 +494,19 @@ def main():
       "vs_baseline": None,
       "dtype": "bf16",
       "data": "synthetic",
-      "config": {
-          "workload": "C3 ragged GQA int8 decode layer-step: KV quantise+stash, ragged attention "
-                      "with fused new token, finalize amortised over 32 layers",
-          "batch": B, "q_heads": HQ, "kv_heads": HKV, "head_dim": D, "max_cache_len": S,
-          "layers_rotated": args.layers, "cached_tokens": r["total_tokens"],
-          "launch": "python" if args.no_graph else "hip graph of one pass over the layers",
-          "kv": "int8 codes + fp32 per-token scales", "lengths": "log-normal(median 400, sigma 1) in [16, 8192], seed 3",
-      },
+      "config": cfg,
       "us_per_layer": round(r["ms_per_step"] * 1e3, 2),
       "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 1),
-      "tokens_per_s": round(B / (r["ms_per_step"] * 1e-3 * LAYERS), 1),
+      "tokens_per_s": round(cfg["batch"] / (r["ms_per_step"] * 1e-3 * model_layers), 1),
       "roofline": {
-          "bound": "hbm", "kernel": "attn_decode_kernel<int8> + attn_merge_kernel (one attention launch)",
+          "bound": "hbm", "kernel": r["kernel"],
           "achieved": round(attn_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
           "frac": round(attn_gbps / HBM_PEAK_GBPS, 4),
-          "traffic": MEASURED_ATTN_TRAFFIC_BYTES if args.layers == LAYERS else None,
-          "us_per_launch": round(r["attn_ms"] * 1e3, 2), "algorithmic_bytes": r["attn_bytes"],
+          "traffic": MEASURED_ATTN_TRAFFIC_BYTES if headline and cfg["layers_rotated"] == LAYERS else None,
+          "us_per_launch": round(r["attn_ms"] * 1e3, 2), "algorithmic_bytes": int(r["attn_bytes"]),
       },
   }
-  if not args.no_cpu_baseline:
+  if headline and not args.no_cpu_baseline:
     line["cpu_baseline"] = run_cpu_baseline()
   print(json.dumps(line))
 

@@ -190,6 +190,14 @@ typedef struct {
   int32_t slot, batch, seq, start; /* dense */
   int32_t total_pages, page_size;  /* paged */
   int32_t in_dtype, dst_dtype, scale_dtype, scale_heads, rounding;
+  /* Several layers in one launch: layer l reads src + l * src_layer_stride and
+   * writes dst + l * dst_layer_stride, scales + l * scale_layer_stride (strides
+   * in elements; stacked tensors).  n_layers 0 or 1 = one layer. */
+  int32_t n_layers;
+  int64_t src_layer_stride, dst_layer_stride, scale_layer_stride;
+  /* Elements between the heads of src; 0 = tokens * dim (contiguous).  Larger
+   * when src is the first `tokens` rows of a longer (heads, T, dim) buffer. */
+  int64_t src_head_stride;
 } jpt_prefill_insert_args;
 
 int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void* stream);

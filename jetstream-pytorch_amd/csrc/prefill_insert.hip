@@ -42,14 +42,17 @@ __global__ void __launch_bounds__(256) prefill_insert_kernel(InsertParams p) {
   const jpt_prefill_insert_args& a = p.a;
   const int t = blockIdx.x;
   const bool is_v = blockIdx.y == 1;
-  const void* src = is_v ? a.src_v : a.src_k;
-  char* dst = static_cast<char*>(is_v ? a.dst_v : a.dst_k);
-  void* scale_out = is_v ? a.v_scale : a.k_scale;
+  const int layer = blockIdx.z;
   const bool paged = a.page_ids != nullptr;
   const bool quant = a.dst_dtype == JPT_I8 && a.in_dtype != JPT_I8;
   const int H = a.heads, D = a.dim, HD = H * D;
   const int esz_in = a.in_dtype == JPT_F32 ? 4 : a.in_dtype == JPT_BF16 ? 2 : 1;
   const int esz_out = quant ? 1 : esz_in;
+  const int esz_scale = a.scale_dtype == JPT_F32 ? 4 : 2;
+  const void* src = static_cast<const char*>(is_v ? a.src_v : a.src_k) + layer * a.src_layer_stride * esz_in;
+  char* dst = static_cast<char*>(is_v ? a.dst_v : a.dst_k) + layer * a.dst_layer_stride * esz_out;
+  void* scale_out = (is_v ? a.v_scale : a.k_scale) == nullptr ? nullptr
+      : static_cast<char*>(is_v ? a.v_scale : a.k_scale) + layer * a.scale_layer_stride * esz_scale;
 
   // destination row of (this token, head h): element index row * D
   int64_t pool_row = 0;  // dense: position in the slot's row; paged: row in the pool
@@ -80,7 +83,8 @@ __global__ void __launch_bounds__(256) prefill_insert_kernel(InsertParams p) {
     }
     return;
   }
-  auto src_index = [&](int h, int d) -> int64_t { return (static_cast<int64_t>(h) * a.tokens + t) * D + d; };
+  const int64_t head_stride = a.src_head_stride > 0 ? a.src_head_stride : static_cast<int64_t>(a.tokens) * D;
+  auto src_index = [&](int h, int d) -> int64_t { return h * head_stride + static_cast<int64_t>(t) * D + d; };
 
   if (!quant) {  // copy
     for (int i = 4 * threadIdx.x; i < HD; i += 4 * blockDim.x) {
@@ -159,6 +163,9 @@ extern "C" int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void*
   JPT_REQUIRE(quant || a.dst_dtype == a.in_dtype, "dst_dtype must be in_dtype (copy) or int8 (quantise)");
   const int esz = a.in_dtype == JPT_F32 ? 4 : a.in_dtype == JPT_BF16 ? 2 : 1;
   JPT_REQUIRE(aligned(a.src_k, 4 * esz) && aligned(a.src_v, 4 * esz), "source rows must be aligned to four elements");
+  JPT_REQUIRE(a.src_head_stride == 0 || (a.src_head_stride >= static_cast<int64_t>(a.tokens) * a.dim && a.src_head_stride % 4 == 0),
+              "src_head_stride must cover the tokens and be a multiple of 4");
+  JPT_REQUIRE(a.src_layer_stride % 4 == 0 && a.dst_layer_stride % 4 == 0, "layer strides must be multiples of 4");
   const int esz_out = quant ? 1 : esz;
   JPT_REQUIRE(aligned(a.dst_k, 4 * esz_out) && aligned(a.dst_v, 4 * esz_out), "destination must be aligned to four elements");
   if (quant) {
@@ -180,7 +187,9 @@ extern "C" int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void*
   }
   if (rows == 0) return JPT_OK;
   InsertParams p{*args};
-  dim3 grid(rows, 2);
+  if (p.a.n_layers <= 0) p.a.n_layers = 1;
+  JPT_REQUIRE(p.a.n_layers <= 65535, "n_layers out of range");
+  dim3 grid(rows, 2, p.a.n_layers);
   if (quant && a.scale_dtype == JPT_BF16)
     hipLaunchKernelGGL(prefill_insert_kernel<true>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), p);
   else

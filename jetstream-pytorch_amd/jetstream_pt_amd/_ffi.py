@@ -66,6 +66,8 @@ class PrefillInsertArgs(_c.Structure):
       ("batch", _i32), ("seq", _i32), ("start", _i32), ("total_pages", _i32),
       ("page_size", _i32), ("in_dtype", _i32), ("dst_dtype", _i32),
       ("scale_dtype", _i32), ("scale_heads", _i32), ("rounding", _i32),
+      ("n_layers", _i32), ("src_layer_stride", _i64), ("dst_layer_stride", _i64),
+      ("scale_layer_stride", _i64), ("src_head_stride", _i64),
   ]
 
 

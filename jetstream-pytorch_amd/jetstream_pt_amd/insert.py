@@ -89,6 +89,32 @@ def insert_prefix_pages_int8(prefix_caches, decode_caches, scale_pages, page_ids
     _ffi.check(_ffi.lib.jpt_prefill_insert(a, _ffi.stream()))
 
 
+def insert_prefix_pages_int8_stacked(prefix_k, prefix_v, pages_k, pages_v, k_scale_pages, v_scale_pages,
+                                     page_ids, *, rounding="rne"):
+  """All layers of one prompt in one launch: prefix_k/v (L, heads, T, D),
+  pages (L, heads, P, ps, D) int8, scale pages (L, Hs, P, ps)."""
+  pk, pv = _ffi.dev(pages_k, "pages_k"), _ffi.dev(pages_v, "pages_v")
+  ks, vs = _ffi.dev(k_scale_pages, "k_scale_pages"), _ffi.dev(v_scale_pages, "v_scale_pages")
+  newk, newv = prefix_k, prefix_v
+  # the first T rows of a longer buffer are taken as they are (no copy)
+  if not (newk.is_cuda and newk.stride(3) == 1 and newk.stride(2) == newk.shape[3] and
+          newk.stride() == newv.stride()):
+    newk, newv = _ffi.dev(newk.contiguous(), "prefix key"), _ffi.dev(newv.contiguous(), "prefix value")
+  layers, heads, total, ps, dim = pk.shape
+  if newk.shape[0] != layers or newk.shape[1] != heads or newk.shape[3] != dim:
+    raise ValueError(f"prefix {tuple(newk.shape)} does not match pages {tuple(pk.shape)}")
+  ids = _ffi.as_i32(page_ids, pk.device)
+  a = _ffi.PrefillInsertArgs(
+      src_k=_ffi.ptr(newk), src_v=_ffi.ptr(newv), dst_k=_ffi.ptr(pk), dst_v=_ffi.ptr(pv),
+      k_scale=_ffi.ptr(ks), v_scale=_ffi.ptr(vs), page_ids=_ffi.ptr(ids), n_pages=ids.numel(),
+      tokens=newk.shape[2], heads=heads, dim=dim, total_pages=total, page_size=ps,
+      in_dtype=_ffi.dtype_code(newk.dtype), dst_dtype=_ffi.I8, scale_dtype=_ffi.dtype_code(ks.dtype),
+      scale_heads=ks.shape[1], rounding=_rounding_code(rounding), n_layers=layers,
+      src_layer_stride=newk.stride(0), dst_layer_stride=pk.stride(0), scale_layer_stride=ks.stride(0),
+      src_head_stride=newk.stride(1))
+  _ffi.check(_ffi.lib.jpt_prefill_insert(a, _ffi.stream()))
+
+
 def insert(env, prefix_caches, prefix_seq_len, caches, cache_scales, slot, *, current_position=0,
            mask=None, start=None, input_pos=None, lens=None):
   """The reference's Engine.insert for dense caches: picks no-wrap or wrap as

@@ -125,3 +125,28 @@ def test_int8_paged_insert_equals_quantise_then_page_layout(tokens):
       want_s[0, page_ids.long(), :] = flat.reshape(n_pages, ps)
       assert torch.equal(dpools[layer][which].cpu(), want)
       assert torch.equal(dscales[layer][which].cpu(), want_s)
+
+
+def test_int8_paged_insert_all_layers_in_one_launch():
+  from jetstream_pt_amd import insert as gins
+  layers, heads, total, ps, dim, tokens = 3, 8, 16, 64, 128, 150
+  g = torch.Generator().manual_seed(5)
+  page_ids = torch.tensor([9, 2, 14], dtype=torch.int32)
+  pk = torch.randint(-127, 128, (layers, heads, total, ps, dim), generator=g, dtype=torch.int8)
+  pv = torch.randint(-127, 128, (layers, heads, total, ps, dim), generator=g, dtype=torch.int8)
+  sk, sv = torch.rand((layers, 1, total, ps), generator=g), torch.rand((layers, 1, total, ps), generator=g)
+  nk = torch.randn((layers, heads, tokens, dim), generator=g).to(torch.bfloat16)
+  nv = torch.randn((layers, heads, tokens, dim), generator=g).to(torch.bfloat16)
+  one = [(pk.to(DEV), pv.to(DEV)), (sk.to(DEV), sv.to(DEV))]
+  per = [[(pk[l].to(DEV), pv[l].to(DEV)) for l in range(layers)], [(sk[l].to(DEV), sv[l].to(DEV)) for l in range(layers)]]
+  # the prompt is the head of a longer buffer: strided rows, no copy
+  longk = torch.cat([nk, torch.ones((layers, heads, 40, dim), dtype=nk.dtype)], dim=2).to(DEV)
+  longv = torch.cat([nv, torch.ones((layers, heads, 40, dim), dtype=nv.dtype)], dim=2).to(DEV)
+  gins.insert_prefix_pages_int8_stacked(longk[:, :, :tokens], longv[:, :, :tokens], one[0][0], one[0][1],
+                                        one[1][0], one[1][1], page_ids)
+  gins.insert_prefix_pages_int8([(nk[l:l + 1].to(DEV), nv[l:l + 1].to(DEV)) for l in range(layers)], per[0], per[1], page_ids)
+  torch.cuda.synchronize()
+  for l in range(layers):
+    assert torch.equal(one[0][0][l], per[0][l][0]) and torch.equal(one[0][1][l], per[0][l][1])
+    assert torch.equal(one[1][0][l], per[1][l][0]) and torch.equal(one[1][1][l], per[1][l][1])
+  assert not torch.equal(one[0][0].cpu(), pk)
