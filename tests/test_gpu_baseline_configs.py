@@ -1,0 +1,217 @@
+"""GPU parity at the full sizes of the five benchmark configurations.
+
+Each test builds the workload exactly as bench.py times it (same shapes, same
+seeded inputs, fewer layers), runs layer-steps through the product path and
+checks every byte the step writes - cache rows, codes, scales, page tables -
+bit for bit against the CPU oracle, the attention output within 1e-2, and that
+nothing else in the cache changed."""
+
+import argparse
+
+import numpy as np
+import pytest
+import torch
+
+import bench
+from oracle import Env as OEnv
+from oracle import attention as oattn
+from oracle import kv_cache as okv
+from oracle import page_manager as opm
+from oracle import quant as oquant
+from oracle.attn_layers import Int8KVAttentionKernel as OInt8Attn
+
+pytestmark = pytest.mark.gpu
+ATOL, RTOL = 1e-2, 1e-2  # attention outputs (bf16), as the reference's own kernel tests use
+
+
+def args(layers):
+  return argparse.Namespace(layers=layers)
+
+
+def close(got, want, rtol=RTOL):
+  got, want = got.float().cpu(), want.float()
+  bad = (got - want).abs() > ATOL + rtol * want.abs()
+  assert not bad.any(), f"{int(bad.sum())} outputs differ, worst {float((got - want).abs().max())}"
+
+
+def test_c1_dense_bf16_eager_update_and_attention():
+  w = bench.build_c1(torch, args(2))
+  cache = w["caches"][0]
+  before_k, before_v = cache.cache_k.clone(), cache.cache_v.clone()
+  out = w["step"](0)
+  torch.cuda.synchronize()
+  pos, b = w["pos"].long(), torch.arange(8)
+  for before, after, new in ((before_k, cache.cache_k, w["xk"]), (before_v, cache.cache_v, w["xv"])):
+    want = before.clone()
+    want[b.to(want.device), :, pos.to(want.device), :] = new[:, :, 0, :]
+    assert torch.equal(after, want)
+  want, _, _ = oattn.closed_form(w["xq"].cpu(), cache.cache_k.cpu(), cache.cache_v.cpu(), mask=w["mask"].cpu())
+  close(out, want)
+
+
+def dense_int8_step_checks(w, batch, hkv):
+  cache, lengths = w["cache"], w["lengths"]
+  nl = cache.cache_k.shape[0]
+  before = [t.clone() for t in (cache.cache_k, cache.cache_v, cache.k_scaler, cache.v_scaler)]
+  out = w["step"](0)
+  torch.cuda.synchronize()
+  # the lazy stash of layer 0: codes and scales of the decode quantiser, computed in float32
+  stash = {}
+  for name, x, codes, scale in (("k", w["xk"], cache.new_ks[0], cache.new_k_scaler[0]),
+                                ("v", w["xv"], cache.new_vs[0], cache.new_v_scaler[0])):
+    want_c, want_s = oquant.quantize_decode(x.cpu(), compute_dtype=torch.float32)
+    assert torch.equal(codes.cpu().reshape(want_c.shape), want_c), name
+    assert torch.equal(scale.cpu().reshape(-1), want_s.reshape(-1)), name
+    stash[name] = (codes.clone(), scale.clone())
+  # attention over cache + merged new token against the oracle's layer kernel
+  oenv = OEnv(batch_size=batch, num_layers=1, ring_buffer=False)
+  ocache = okv.Int8KVCacheGenerate.empty((1, batch, hkv, cache.cache_k.shape[3], bench.D), None, oenv,
+                                         scale_dtype=torch.float32)
+  ocache.cache_k, ocache.cache_v = before[0][:1].cpu(), before[1][:1].cpu()
+  ocache.k_scaler, ocache.v_scaler = before[2][:1].cpu(), before[3][:1].cpu()
+  ocache.input_pos = lengths
+  want = OInt8Attn(oenv, 0)(w["xq"].cpu(), w["xk"].cpu(), w["xv"].cpu(), None, ocache, start=None, end=lengths)
+  # the reference recurrence rounds the running output to bf16 after every block of 512
+  # positions, so on long slots it strays a few bf16 steps from the exact result
+  close(out, want, rtol=4 * 2.0 ** -7)
+  # and slot by slot against the float64 closed form over cache ++ new token
+  seq = cache.cache_k.shape[3]
+  for b in range(batch):
+    n = int(lengths[b])
+    if n >= seq:
+      continue
+    k = torch.cat([before[0][0, b, :, :n], stash["k"][0].reshape(batch, hkv, 1, bench.D)[b]], dim=1).cpu()
+    v = torch.cat([before[1][0, b, :, :n], stash["v"][0].reshape(batch, hkv, 1, bench.D)[b]], dim=1).cpu()
+    ks = torch.cat([before[2][0, b, 0, :n, 0], stash["k"][1].reshape(batch)[b:b + 1]]).reshape(1, 1, n + 1, 1).cpu()
+    vs = torch.cat([before[3][0, b, 0, :n, 0], stash["v"][1].reshape(batch)[b:b + 1]]).reshape(1, 1, n + 1, 1).cpu()
+    exact, _, _ = oattn.closed_form(w["xq"][b:b + 1].cpu(), k[None], v[None], k_scale=ks, v_scale=vs)
+    close(out[b:b + 1], exact)
+  # the remaining layers, then finalize(): every layer's row pos[b] holds its stash, nothing else moved
+  stashes = [stash]
+  for i in range(1, nl):
+    w["step"](i)
+    if i < nl - 1:
+      stashes.append({"k": (cache.new_ks[i].clone(), cache.new_k_scaler[i].clone()),
+                      "v": (cache.new_vs[i].clone(), cache.new_v_scaler[i].clone())})
+  torch.cuda.synchronize()
+  pos = lengths.long().to(cache.cache_k.device)
+  b = torch.arange(batch, device=pos.device)
+  ok = pos < cache.cache_k.shape[3]  # a full slot has no row left: nothing is written for it
+  for l, st in enumerate(stashes):
+    for which, (codes, scale) in (("k", st["k"]), ("v", st["v"])):
+      want_c = before[0 if which == "k" else 1][l].clone()
+      want_c[b[ok], :, pos[ok], :] = codes.reshape(batch, hkv, bench.D)[ok]
+      got_c = (cache.cache_k if which == "k" else cache.cache_v)[l]
+      assert torch.equal(got_c, want_c), (l, which)
+      want_s = before[2 if which == "k" else 3][l].clone()
+      want_s[b[ok], 0, pos[ok], 0] = scale.reshape(batch)[ok]
+      got_s = (cache.k_scaler if which == "k" else cache.v_scaler)[l]
+      assert torch.equal(got_s, want_s), (l, which)
+
+
+def test_c2_int8_mha_decode_step():
+  dense_int8_step_checks(bench.build_c2(torch, args(2)), 96, 32)
+
+
+def test_c3_ragged_gqa_int8_decode_step():
+  dense_int8_step_checks(bench.build_c3(torch, args(2)), 128, 8)
+
+
+def replay_manager(w, seed, total, ps, max_pages, batch):
+  """The same allocator calls on the oracle's manager; returns it after
+  checking every index array the product handed out."""
+  rng = np.random.default_rng(seed)
+  om = opm.PageAttentionManager(batch, total, ps, max_pages, free_list_order=rng.permutation(total))
+  for slot in range(batch):
+    om.reserve_pages_insert(slot, int(w["initial_lengths"][slot]))
+  for entry in w["state"]["log"]:
+    if entry[0] == "insert":
+      _, slot, n, ids = entry
+      om.free_pages_resource(slot)
+      num, view = om.reserve_pages_insert(slot, n)
+      assert np.array_equal(np.asarray(view[:num]), ids)
+    else:
+      _, lens, idx = entry
+      om.fill_new_pages(lens)
+      assert np.array_equal(om.get_page_token_indices(lens), idx)
+  pam = w["pam"]
+  assert np.array_equal(om.page_indices, pam.page_indices)
+  assert np.array_equal(om.lengths, pam.lengths)
+  return om
+
+
+def paged_attention_subset(w, out, layer, slots, int8):
+  pk, pv = w["pools"][0][layer], w["pools"][1][layer]
+  pam, ps = w["pam"], pk.shape[2]
+  for b in slots:
+    n = int(pam.lengths[b])
+    pages = torch.from_numpy(pam.page_indices[b, : (n + ps - 1) // ps].astype(np.int64)).to(pk.device)
+    k = pk[:, pages].reshape(pk.shape[0], -1, bench.D)[:, :n].cpu()
+    v = pv[:, pages].reshape(pk.shape[0], -1, bench.D)[:, :n].cpu()
+    ks = vs = None
+    if int8:
+      sk, sv = w["scale_pages"][0][layer], w["scale_pages"][1][layer]
+      ks = sk[:, pages].reshape(1, 1, -1, 1)[:, :, :n].cpu()
+      vs = sv[:, pages].reshape(1, 1, -1, 1)[:, :, :n].cpu()
+    want, _, _ = oattn.closed_form(w["xq"][b:b + 1].cpu(), k[None], v[None], k_scale=ks, v_scale=vs, sm_scale=1.0)
+    close(out[b:b + 1], want)
+
+
+def test_c4_paged_bf16_decode_steps():
+  w = bench.build_c4(torch, args(1))
+  pk, pv = w["pools"][0][0], w["pools"][1][0]
+  want_k, want_v = pk.clone(), pv.clone()
+  out = None
+  for i in range(2):  # two decode steps of the one layer
+    out = w["step"](i)
+  torch.cuda.synchronize()
+  replay_manager(w, 4, 32768, 64, 128, 256)
+  for entry in w["state"]["log"]:
+    idx = torch.from_numpy(entry[2]).long().to(pk.device)
+    pages, toks, slots = idx[0], idx[1] % 64, idx[2]
+    want_k[:, pages, toks, :] = w["xk"][slots, :, 0, :].transpose(0, 1)
+    want_v[:, pages, toks, :] = w["xv"][slots, :, 0, :].transpose(0, 1)
+  assert torch.equal(pk, want_k) and torch.equal(pv, want_v)
+  paged_attention_subset(w, out, 0, range(0, 256, 11), int8=False)
+
+
+def test_c5_paged_int8_prompt_churn_and_decode_steps():
+  nl = 2
+  w = bench.build_c5(torch, args(nl))
+  pools, scales = w["pools"], w["scale_pages"]
+  want = [[t[l].clone() for t in (pools[0], pools[1], scales[0], scales[1])] for l in range(nl)]
+  out = None
+  for i in range(2 * nl):  # two decode steps over both layers
+    o = w["step"](i)
+    if i % nl == 0:
+      out = o
+  torch.cuda.synchronize()
+  replay_manager(w, 5, 16384, 64, 64, 256)
+  dev = pools[0].device
+  dk, sk_new = oquant.quantize_decode(w["xk"].cpu(), compute_dtype=torch.float32)
+  dv, sv_new = oquant.quantize_decode(w["xv"].cpu(), compute_dtype=torch.float32)
+  for entry in w["state"]["log"]:
+    for l in range(nl):
+      wk, wv, wsk, wsv = want[l]
+      if entry[0] == "insert":
+        _, slot, n, ids = entry
+        pages = torch.from_numpy(ids.astype(np.int64)).to(dev)
+        for src, wc, ws in ((w["prompts"][0], wk, wsk), (w["prompts"][1], wv, wsv)):
+          codes, sc = oquant.quantize_insert(src[l, :, :n].cpu()[None], compute_dtype=torch.float32)
+          padded = torch.zeros((8, len(ids) * 64, bench.D), dtype=torch.int8)
+          padded[:, :n] = codes[0]
+          wc[:, pages] = padded.reshape(8, len(ids), 64, bench.D).to(dev)
+          flat = ws[0, pages].reshape(-1)
+          flat[:n] = sc.reshape(-1).to(dev)
+          ws[0, pages] = flat.reshape(len(ids), 64)
+      else:
+        idx = torch.from_numpy(entry[2]).long().to(dev)
+        pages, toks, slots = idx[0], idx[1] % 64, idx[2]
+        wk[:, pages, toks, :] = dk.to(dev)[slots, :, 0, :].transpose(0, 1)
+        wv[:, pages, toks, :] = dv.to(dev)[slots, :, 0, :].transpose(0, 1)
+        wsk[0, pages, toks] = sk_new.to(dev).reshape(-1)[slots]
+        wsv[0, pages, toks] = sv_new.to(dev).reshape(-1)[slots]
+  for l in range(nl):
+    for got, exp, name in zip((pools[0][l], pools[1][l], scales[0][l], scales[1][l]), want[l], "k v ks vs".split()):
+      assert torch.equal(got, exp), (l, name)
+  paged_attention_subset(w, out, 0, range(0, 256, 11), int8=True)
