@@ -52,6 +52,9 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef const __attribute__((address_space(1))) void* global_ptr;
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
+#ifndef JPT_ATTN_EXPERIMENT_CUT
+#define JPT_ATTN_EXPERIMENT_CUT 0  // development: stop a tile's work early (timing experiments only)
+#endif
 #ifndef JPT_ATTN_CONSUMERS
 #define JPT_ATTN_CONSUMERS 3
 #endif
@@ -128,6 +131,12 @@ __device__ __forceinline__ i32x4 lds_peek4(const int* p) {
 __device__ __forceinline__ void lds_poke(int* p, int v) {
   const uint32_t addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_int_ptr)p));
   asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(v) : "memory");
+}
+
+// An LDS word every lane reads alike, as a wave-uniform (scalar) value: what
+// the producer branches on stays out of the vector condition path.
+__device__ __forceinline__ int lds_peek_uniform(const int* p) {
+  return __builtin_amdgcn_readfirstlane(lds_peek(p));
 }
 
 // Load through the scalar data path.  `p` must be the same in every lane and
@@ -295,14 +304,17 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   __shared__ int sm_arrived_all[kGroups][C::kFoldBufs];
   __shared__ int sm_folded_all[kGroups][C::kFoldBufs];
   __shared__ int sm_abort;
+  JPT_TR(__shared__ int sm_issue_time[kGroups][C::kSlots];)
   __shared__ __attribute__((aligned(16))) int sm_items_all[kGroups][kListedItems][8];
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int hw_wave = tid >> 6;
+  const int hw_wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, and known to be
   const int group = hw_wave / kGroupWaves;
   // role index: consumers 0..kConsumers-1, producer kConsumers
   const int wave = hw_wave % kGroupWaves == 0 ? kConsumers : hw_wave % kGroupWaves - 1;
   JPT_TR(const unsigned long long tr_start = __builtin_amdgcn_s_memrealtime();)
+  JPT_TR(unsigned long long* tr_line = (p.trace && blockIdx.x == 5 && group == 0 && lane == 0) ? p.trace + 1024 * 16 * 8 : nullptr;)
+  JPT_TR(unsigned long long tr_sig = 0; int tr_polls = 0;)
   JPT_TR(unsigned long long tr_wait = 0; unsigned long long tr_fold = 0; unsigned long long tr_first = 0; unsigned long long tr_t = 0; int tr_tiles = 0;)
   for (int i = tid; i < kGroups * C::kSlots; i += kThreads) {
     (&sm_filled_all[0][0])[i] = 0;
@@ -457,7 +469,9 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       while (signalled < issued) {
         const int need = sig_base + C::kLoadsPerTile + (((carries_q >> (signalled & 63)) & 1) ? q_loads : 0);
         if (done < need) break;
-        if (lane == 0) lds_poke(&sm_filled[sig_slot], sig_round);
+        lds_poke(&sm_filled[sig_slot], sig_round);  // every lane stores the same word
+        JPT_TR(tr_fold += static_cast<unsigned>(static_cast<int>(__builtin_amdgcn_s_memrealtime()) - lds_peek(&sm_issue_time[group][sig_slot]));)
+        JPT_TR(if (tr_line && signalled < 256) tr_line[signalled * 8 + 2] = __builtin_amdgcn_s_memrealtime();)
         sig_base = need;
         carries_q &= ~(1ull << (signalled & 63));
         ++signalled;
@@ -468,9 +482,11 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     // `room` more loads fit under the load counter's limit of 63.
     auto wait_counter = [&](int* counter, int needed, int room) -> bool {
       for (int spins = 0;; ++spins) {
+        JPT_TR(const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();)
         signal_landed();
-        if (loads_issued - sig_base + room <= 63 && lds_peek(counter) >= needed) return true;
-        if (spins > kSpinLimit || lds_peek(&sm_abort)) {
+        JPT_TR(tr_sig += __builtin_amdgcn_s_memrealtime() - t0; ++tr_polls;)
+        if (loads_issued - sig_base + room <= 63 && lds_peek_uniform(counter) >= needed) return true;
+        if (spins > kSpinLimit || lds_peek_uniform(&sm_abort)) {
           lds_poke(&sm_abort, 1);
           __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
           return false;
@@ -556,9 +572,12 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         // wait for the slot's previous tile to be taken, handing over landed
         // tiles meanwhile
         JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
+        JPT_TR(if (tr_line && issued < 256) tr_line[issued * 8 + 0] = tr_t;)
         if (!wait_counter(&sm_freed[fill_slot], fill_round, C::kLoadsPerTile)) return;
+        JPT_TR(if (tr_line && issued < 256) tr_line[issued * 8 + 1] = __builtin_amdgcn_s_memrealtime();)
         JPT_TR(tr_wait += __builtin_amdgcn_s_memrealtime() - tr_t; if (!tr_first) tr_first = __builtin_amdgcn_s_memrealtime() - tr_start;)
         char* slot = ring + fill_slot * C::kSlotBytes;
+        JPT_TR(lds_poke(&sm_issue_time[group][fill_slot], static_cast<int>(__builtin_amdgcn_s_memrealtime()));)
 #pragma unroll
         for (int j = 0; j < kLoadsPerMatrix; ++j) {
           const uint32_t off = static_cast<uint32_t>(min(row_of[j], valid - 1)) * C::kRowBytes + piece_off[j];
@@ -587,7 +606,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     }
     for (int spins = 0; signalled < issued; ++spins) {
       signal_landed();
-      if (spins > kSpinLimit || lds_peek(&sm_abort)) {
+      if (spins > kSpinLimit || lds_peek_uniform(&sm_abort)) {
         lds_poke(&sm_abort, 1);
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
         return;
@@ -596,8 +615,8 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     }
     JPT_TR(if (p.trace && lane == 0) {
       unsigned long long* o = p.trace + (static_cast<size_t>(blockIdx.x) * kWaves + hw_wave) * 8;
-      o[0] = issued; o[1] = tr_wait; o[2] = 0; o[3] = __builtin_amdgcn_s_memrealtime() - tr_start;
-      o[4] = tr_start; o[5] = 0; o[6] = tr_first; o[7] = (__builtin_amdgcn_s_getreg(0xF804) >> 4) & 3;
+      o[0] = issued; o[1] = tr_wait; o[2] = tr_fold; o[3] = __builtin_amdgcn_s_memrealtime() - tr_start;
+      o[4] = tr_start; o[5] = 0; o[6] = tr_first; o[7] = (static_cast<unsigned long long>(tr_polls) << 32) | tr_sig;
     })
     return;
   }
@@ -629,6 +648,11 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
     if (!wait_for(&sm_filled[s], t / C::kSlots + 1)) return false;
     JPT_TR(tr_wait += __builtin_amdgcn_s_memrealtime() - tr_t; ++tr_tiles; if (!tr_first) tr_first = __builtin_amdgcn_s_memrealtime() - tr_start;)
+#ifdef JPT_ATTN_EXPERIMENT_NO_COMPUTE
+    if (lane == 0)
+      __hip_atomic_fetch_add(&sm_freed[s], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    return true;
+#endif
     const char* slot = ring + s * C::kSlotBytes;
     const char* side = slot + 2 * C::kTileBytes;
     T tile;
@@ -672,12 +696,31 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     if (lane == 0)
       __hip_atomic_fetch_add(&sm_freed[s], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
 
+#if JPT_ATTN_EXPERIMENT_CUT == 1
+    {
+      uint32_t keep = 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) keep ^= tile.v[i].x ^ tile.v[i].y;
+      keep ^= tile.ka[0].x ^ tile.ka[1].w ^ tile.kb[0].y ^ tile.kb[1].z ^ __float_as_uint(ks[0] + vs[7]);
+      asm volatile("" ::"v"(keep));
+      return true;
+    }
+#endif
     f32x4 sa = s_init, sb = s_init;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
       sa = T::mfma(tile.k_op(false, kk), qop[kk], sa);
       sb = T::mfma(tile.k_op(true, kk), qop[kk], sb);
     }
+#if JPT_ATTN_EXPERIMENT_CUT == 2
+    {
+      uint32_t keep = 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) keep ^= tile.v[i].x ^ tile.v[i].y;
+      asm volatile("" ::"v"(keep), "v"(sa), "v"(sb), "v"(ks[0] + vs[7]));
+      return true;
+    }
+#endif
     float sc[8];
     float tmax = -INFINITY;
 #pragma unroll
