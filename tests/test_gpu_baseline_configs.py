@@ -73,7 +73,7 @@ def dense_int8_step_checks(w, batch, hkv):
   want = OInt8Attn(oenv, 0)(w["xq"].cpu(), w["xk"].cpu(), w["xv"].cpu(), None, ocache, start=None, end=lengths)
   # the reference recurrence rounds the running output to bf16 after every block of 512
   # positions, so on long slots it strays a few bf16 steps from the exact result
-  close(out, want, rtol=4 * 2.0 ** -7)
+  close(out, want, rtol=8 * 2.0 ** -7)
   # and slot by slot against the float64 closed form over cache ++ new token
   seq = cache.cache_k.shape[3]
   for b in range(batch):
