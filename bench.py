@@ -123,15 +123,16 @@ def build_dense_int8(torch, nl, batch, hq, hkv, seq, lengths, name):
 
   plan, _ = ak.precompute_ragged_block_indices(pos, batch, hq, hkv, seq)
   new = dict(new_key=cache.new_ks[0], new_value=cache.new_vs[0],
-             new_k_scaler=cache.new_k_scaler[0], new_v_scaler=cache.new_v_scaler[0])
+             new_k_scaler=cache.new_k_scaler[0], new_v_scaler=cache.new_v_scaler[0],
+             new_key_raw=xk, new_value_raw=xv)  # the launch quantises the token too, as in step()
 
   def attn_only(i):
     return ak.ragged_mha(xq, cache.cache_k, cache.cache_v, i % nl, None, plan.lengths, plan, None,
                          cache.k_scaler, cache.v_scaler, **new)
 
   total = int(lengths.sum())
-  ab = dense_attn_bytes(total, batch, hq, hkv, 1, True, True)
   append = batch * hkv * D * (2 + 1) * 2 + batch * 4 * 2           # bf16 in, codes + fp32 scales out
+  ab = dense_attn_bytes(total, batch, hq, hkv, 1, True, True)
   finalize = (batch * hkv * D + batch * 4) * 2 * 2                # per layer: stash read, cache written
   return dict(step=step, attn_only=attn_only, step_bytes=ab + append + finalize, attn_bytes=ab, graph=True,
               cache=cache, lengths=lengths, xq=xq, xk=xk, xv=xv, env=env,

@@ -236,6 +236,15 @@ int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void* stream);
  * lazy-update mode with a second flash_attention call and seven elementwise
  * ops (layers.py:534-550, :702-718).
  *
+ * new_k_raw/new_v_raw: NULL, or the new token before quantisation,
+ * (batch, kv_heads, 1, dim) bf16, for an int8 cache.  The call then also does
+ * the work of jpt_kv_append_quant_i8 for that token (Int8KVCacheGenerate.update's
+ * quantize, cache_manager.py:532-537, 606-633): new_k/new_v and
+ * new_k_scale/new_v_scale become OUTPUTS that receive its codes and scales
+ * (bit-identical to jpt_kv_append_quant_i8 with `new_rounding`), and the token is
+ * attended with them.  One launch less per layer; the reference has the
+ * quantiser and the attention as separate XLA ops.
+ *
  * workspace: device scratch of at least jpt_attn_workspace_bytes(args)
  * bytes, 256-byte aligned.  Its first JPT_ATTN_WS_STATE_BYTES must be zero
  * before the first call and are left zero by every call; calls sharing one
@@ -274,6 +283,9 @@ typedef struct {
                             these lengths (same batch, heads and lengths as the
                             previous call on this workspace): skip planning.
                             A decode step plans once and reuses it per layer. */
+  const void* new_k_raw; /* see above; both or neither */
+  const void* new_v_raw;
+  int32_t new_rounding;  /* JPT_ROUND_* of the fused quantiser */
 } jpt_attn_args;
 
 int64_t jpt_attn_workspace_bytes(const jpt_attn_args* args);

@@ -53,7 +53,7 @@ int32_t persistent_blocks() {
   static int32_t v = [] {
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) == hipSuccess)
-      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+      if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cus = 256;
     const int32_t per_cu = env_int("JPT_ATTN_BLOCKS_PER_CU", 2);
     return (cus * per_cu + 7) / 8 * 8;
   }();
@@ -224,6 +224,8 @@ bool attn_fast_supported(const jpt_attn_args& a, AttnMode mode) {
   if (a.k_scale && (!aligned(a.k_scale, 16) || !aligned(a.v_scale, 16))) return false;
   if (!aligned(a.q, 16) || !aligned(a.k, 16) || !aligned(a.v, 16)) return false;
   if (a.new_k && (!aligned(a.new_k, 16) || !aligned(a.new_v, 16))) return false;
+  // the new token's raw rows of all heads must fit a tile's key area
+  if (a.new_k_raw && (a.kv_heads > 16 || !aligned(a.new_k_raw, 16) || !aligned(a.new_v_raw, 16))) return false;
   return true;
 }
 
@@ -304,7 +306,29 @@ static int32_t attn_entry(const jpt_attn_args* args, jpt::AttnMode mode, void* s
   if (st != JPT_OK) return st;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (attn_fast_supported(*args, mode)) return attn_fast_launch(*args, mode, s);
-  return attn_generic_launch(*args, mode, s);
+  jpt_attn_args a = *args;
+  if (a.new_k_raw) {  // no fused quantiser on this route: quantise first, then attend the codes
+    jpt_quant_append_args q{};
+    q.new_k = a.new_k_raw;
+    q.new_v = a.new_v_raw;
+    q.out_k = const_cast<void*>(a.new_k);
+    q.out_v = const_cast<void*>(a.new_v);
+    q.out_k_scale = const_cast<void*>(a.new_k_scale);
+    q.out_v_scale = const_cast<void*>(a.new_v_scale);
+    q.batch = a.batch;
+    q.heads = a.kv_heads;
+    q.dim = a.dim;
+    q.seq = 1;
+    q.in_dtype = JPT_BF16;
+    q.scale_dtype = a.scale_dtype;
+    q.scale_heads = a.scale_heads;
+    q.rounding = a.new_rounding;
+    st = jpt_kv_append_quant_i8(&q, stream);
+    if (st != JPT_OK) return st;
+    a.new_k_raw = a.new_v_raw = nullptr;
+    if (attn_fast_supported(a, mode)) return attn_fast_launch(a, mode, s);
+  }
+  return attn_generic_launch(a, mode, s);
 }
 
 int32_t jpt_attn_plan(const jpt_attn_args* args, int32_t paged, void* stream) {

@@ -314,7 +314,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   const int wave = hw_wave % kGroupWaves == 0 ? kConsumers : hw_wave % kGroupWaves - 1;
   JPT_TR(const unsigned long long tr_start = __builtin_amdgcn_s_memrealtime();)
   JPT_TR(unsigned long long* tr_line = (p.trace && blockIdx.x == 5 && group == 0 && lane == 0) ? p.trace + 1024 * 16 * 8 : nullptr;)
-  JPT_TR(unsigned long long tr_sig = 0; int tr_polls = 0;)
+  JPT_TR(unsigned long long tr_sig = 0; int tr_polls = 0; unsigned long long tr_qwait = 0;)
   JPT_TR(unsigned long long tr_wait = 0; unsigned long long tr_fold = 0; unsigned long long tr_first = 0; unsigned long long tr_t = 0; int tr_tiles = 0;)
   for (int i = tid; i < kGroups * C::kSlots; i += kThreads) {
     (&sm_filled_all[0][0])[i] = 0;
@@ -334,6 +334,8 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   const int worker = static_cast<int>(blockIdx.x) + group * static_cast<int>(gridDim.x);
   const int n_rounds = (p.total_items + G - 1) / G;
   const bool has_new = a.new_k != nullptr;
+  // the new token arrives unquantised: the consumer of its tile quantises it
+  const bool quant_new = std::is_same<KV, int8_t>::value && a.new_k_raw != nullptr;
 
   // Item of round k of this worker: virtual ids k*G + j with j running forwards
   // in even rounds and backwards in odd ones, so that with entries sorted
@@ -536,31 +538,42 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         vt = static_cast<const char*>(a.v) + row0 * C::kRowBytes;
         srow = (static_cast<int64_t>(cur.slot) * a.scale_heads + hs) * a.seq + cur.start;
       }
+      // the step's new token is the item's first tile: the consumer that gets it
+      // has the rest of the item to make up for the extra work it can carry
+      const int n_new = nt - n_cache;
       for (int ti = 0; ti < nt; ++ti) {
-        const bool is_new = ti >= n_cache;
+        const bool is_new = ti < n_new;
+        const int ct = ti - n_new;  // tile of the cache
         int valid = 1;  // the new token: every row of the tile is that one token
         const char* sc_src = scale_lane;
+        const char *tk = kt, *tv = vt;
+        int64_t ts = srow;
         if (is_new) {
           const int64_t row = static_cast<int64_t>(cur.slot) * a.kv_heads + cur.h;
-          kt = static_cast<const char*>(a.new_k) + row * C::kRowBytes;
-          vt = static_cast<const char*>(a.new_v) + row * C::kRowBytes;
+          tk = static_cast<const char*>(a.new_k) + row * C::kRowBytes;
+          tv = static_cast<const char*>(a.new_v) + row * C::kRowBytes;
+          if (quant_new) {  // the bf16 rows of all the slot's heads, copied as they lie
+            const int64_t raw = static_cast<int64_t>(cur.slot) * a.kv_heads * (kD * 2);
+            tk = static_cast<const char*>(a.new_k_raw) + raw;
+            tv = static_cast<const char*>(a.new_v_raw) + raw;
+          }
           // float32 scales of the new token come through the ring like any
           // tile's; bf16 ones are read by the consumer, and the tile loads the
           // head of the scale tensors only to keep its load count
-          srow = 0;
+          ts = 0;
           if (SCALE == kScaleF32) {
             sc_src = new_scale_lane;
-            srow = static_cast<int64_t>(cur.slot) * a.scale_heads + hs;
+            ts = static_cast<int64_t>(cur.slot) * a.scale_heads + hs;
           }
         } else {
-          const int t0 = cur.start + ti * kTile;
+          const int t0 = cur.start + ct * kTile;
           valid = min(kTile, cur.start + cur.count - t0);
           if (PAGED) {  // a tile never straddles a page
             const int64_t in_pool = static_cast<int64_t>(page) * a.page_size + t0 % a.page_size;
             const int64_t row0 = static_cast<int64_t>(cur.h) * a.total_pages * a.page_size + in_pool;
-            kt = static_cast<const char*>(a.k) + row0 * C::kRowBytes;
-            vt = static_cast<const char*>(a.v) + row0 * C::kRowBytes;
-            srow = static_cast<int64_t>(hs) * a.total_pages * a.page_size + in_pool;
+            tk = static_cast<const char*>(a.k) + row0 * C::kRowBytes;
+            tv = static_cast<const char*>(a.v) + row0 * C::kRowBytes;
+            ts = static_cast<int64_t>(hs) * a.total_pages * a.page_size + in_pool;
             // page of the next tile, read while this one is issued
             const int tn = min(t0 + kTile, cur.start + cur.count - 1);
             page = load_uniform(a.page_table + (static_cast<int64_t>(cur.slot) * a.max_pages + tn / a.page_size));
@@ -580,24 +593,25 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         JPT_TR(lds_poke(&sm_issue_time[group][fill_slot], static_cast<int>(__builtin_amdgcn_s_memrealtime()));)
 #pragma unroll
         for (int j = 0; j < kLoadsPerMatrix; ++j) {
-          const uint32_t off = static_cast<uint32_t>(min(row_of[j], valid - 1)) * C::kRowBytes + piece_off[j];
-          __builtin_amdgcn_global_load_lds((global_ptr)(kt + off), (lds_ptr)(slot + j * 1024), 16, 0, 0);
-          __builtin_amdgcn_global_load_lds((global_ptr)(vt + off), (lds_ptr)(slot + C::kTileBytes + j * 1024), 16, 0, 0);
+          uint32_t off = static_cast<uint32_t>(min(row_of[j], valid - 1)) * C::kRowBytes + piece_off[j];
+          if (is_new && quant_new) off = static_cast<uint32_t>(min(64 * j + lane, a.kv_heads * (kD / 8) - 1)) * 16;
+          __builtin_amdgcn_global_load_lds((global_ptr)(tk + off), (lds_ptr)(slot + j * 1024), 16, 0, 0);
+          __builtin_amdgcn_global_load_lds((global_ptr)(tv + off), (lds_ptr)(slot + C::kTileBytes + j * 1024), 16, 0, 0);
         }
         char* side = slot + 2 * C::kTileBytes;
         if (SCALE) {
           if (lane < 2 * kHalf)
-            __builtin_amdgcn_global_load_lds((global_ptr)(sc_src + srow * kEs), (lds_ptr)side, 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((global_ptr)(sc_src + ts * kEs), (lds_ptr)side, 4, 0, 0);
         }
         if (MASK) {
-          const float* src = static_cast<const float*>(a.mask) + cur.slot * a.mask_stride_b + (is_new ? 0 : cur.start + ti * kTile);
+          const float* src = static_cast<const float*>(a.mask) + cur.slot * a.mask_stride_b + (is_new ? 0 : cur.start + ct * kTile);
           if (lane < kTile)
             __builtin_amdgcn_global_load_lds((global_ptr)(src + lane), (lds_ptr)(side + 256), 4, 0, 0);
         }
         ++issued;
         loads_issued += C::kLoadsPerTile;
         if (++fill_slot == C::kSlots) { fill_slot = 0; ++fill_round; }
-        if (!PAGED) {
+        if (!PAGED && !is_new) {
           kt += kTile * C::kRowBytes;
           vt += kTile * C::kRowBytes;
           srow += kTile;
@@ -642,6 +656,54 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   // accumulates it; `valid` positions of the tile count (all of them when
   // `full_tag` says so).
   int cur_slot = 0, cur_h = 0;  // of the item being consumed
+  // Quantises the new token of slot cur_slot, whose kv_heads bf16 rows lie one
+  // after another in `area` (the tile's key or value area): arithmetic and
+  // rounding of jpt_kv_append_quant_i8, each step rounded to the scale dtype.
+  // The absmax runs over every head (one scale per token) or over head cur_h;
+  // only head cur_h is coded, two elements a lane.  Its codes replace row 0 of
+  // the area, in tile layout, and go to the stash; the item of head 0 (every
+  // item, with per-head scales) stores the scale.
+  auto quantise_new = [&](char* area, int8_t* stash, void* scale_out) -> float {
+    constexpr bool kBf16Math = SCALE == kScaleBF16;
+    auto rnd = [](float x) { return kBf16Math ? round_to_bf16(x) : x; };
+    const uint32_t pair = *reinterpret_cast<const uint32_t*>(area + cur_h * (kD * 2) + lane * 4);
+    const float x0 = __uint_as_float(pair << 16), x1 = __uint_as_float(pair & 0xffff0000u);
+    float m = fmaxf(fabsf(x0), fabsf(x1));
+    if (a.scale_heads == 1) {
+      for (int at = lane * 32; at < a.kv_heads * (kD * 2); at += 64 * 32) {
+        const uint4 r0 = *reinterpret_cast<const uint4*>(area + at);
+        const uint4 r1 = *reinterpret_cast<const uint4*>(area + at + 16);
+        const uint32_t raw[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          m = fmaxf(m, fmaxf(fabsf(__uint_as_float(raw[i] << 16)), fabsf(__uint_as_float(raw[i] & 0xffff0000u))));
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    if (a.new_rounding == JPT_ROUND_RNE) m = fmaxf(m, rnd(1e-5f));
+    const float sc = rnd(m / 127.0f);
+    int c0, c1;
+    if (a.new_rounding == JPT_ROUND_TRUNC) {
+      const float q0 = rnd(x0 / sc), q1 = rnd(x1 / sc);
+      c0 = (q0 != q0) ? 0 : static_cast<int>(q0);  // 0/0 -> 0; the cast truncates
+      c1 = (q1 != q1) ? 0 : static_cast<int>(q1);
+    } else {
+      const float inv = rnd(1.0f / sc);
+      c0 = static_cast<int>(fminf(fmaxf(rintf(rnd(x0 * inv)), -128.f), 127.f));
+      c1 = static_cast<int>(fminf(fmaxf(rintf(rnd(x1 * inv)), -128.f), 127.f));
+    }
+    const uint16_t codes = static_cast<uint16_t>((c0 & 0xff) | ((c1 & 0xff) << 8));
+    // row 0 of the tile: piece p sits at piece slot p ^ 0.  Every lane has read
+    // its raw elements above, before any lane's codes land on them.
+    *reinterpret_cast<uint16_t*>(area + lane * 2) = codes;
+    *reinterpret_cast<uint16_t*>(stash + (static_cast<int64_t>(cur_slot) * a.kv_heads + cur_h) * kD + lane * 2) = codes;
+    if (lane == 0 && (a.scale_heads != 1 || cur_h == 0)) {
+      const int64_t si = static_cast<int64_t>(cur_slot) * a.scale_heads + (a.scale_heads == 1 ? 0 : cur_h);
+      store_from_f32(scale_out, si, kBf16Math ? JPT_BF16 : JPT_F32, sc);
+    }
+    return sc;
+  };
   auto consume_tile = [&](int t, int valid, bool is_new, auto full_tag) -> bool {
     constexpr bool FULL = decltype(full_tag)::value;
     const int s = t % C::kSlots;
@@ -653,8 +715,14 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       __hip_atomic_fetch_add(&sm_freed[s], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     return true;
 #endif
-    const char* slot = ring + s * C::kSlotBytes;
+    char* slot = ring + s * C::kSlotBytes;
     const char* side = slot + 2 * C::kTileBytes;
+    float new_ks = 0.f, new_vs = 0.f;
+    const bool quant_here = !FULL && is_new && quant_new;
+    if (quant_here) {
+      new_ks = quantise_new(slot, static_cast<int8_t*>(const_cast<void*>(a.new_k)), const_cast<void*>(a.new_k_scale));
+      new_vs = quantise_new(slot + C::kTileBytes, static_cast<int8_t*>(const_cast<void*>(a.new_v)), const_cast<void*>(a.new_v_scale));
+    }
     T tile;
     tile.read(slot, slot + C::kTileBytes, r, g, pos);
     // the lane's positions are 4g..4g+3 and 16+4g..16+4g+3
@@ -681,6 +749,10 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       vs[2] = __uint_as_float(v0.y << 16); vs[3] = __uint_as_float(v0.y & 0xffff0000u);
       vs[4] = __uint_as_float(v1.x << 16); vs[5] = __uint_as_float(v1.x & 0xffff0000u);
       vs[6] = __uint_as_float(v1.y << 16); vs[7] = __uint_as_float(v1.y & 0xffff0000u);
+    }
+    if (quant_here) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) { ks[i] = new_ks; vs[i] = new_vs; }
     }
     if (MASK) {
       const float4* smk = reinterpret_cast<const float4*>(side + 256);
@@ -847,7 +919,9 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     const int n_cache = cache_tiles(cur), nt = item_tiles(cur);
     if (nt > 0) {
       // query rows: staged by the producer ahead of the item's first tile
+      JPT_TR(const unsigned long long tq0 = __builtin_amdgcn_s_memrealtime();)
       if (!wait_for(&sm_filled[base % C::kSlots], base / C::kSlots + 1)) return;
+      JPT_TR(tr_qwait += __builtin_amdgcn_s_memrealtime() - tq0;)
       const int qb = q_seq++ % C::kQBufs;
       uint4 u[4];
 #pragma unroll
@@ -910,8 +984,8 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     l_run = 0.f;
     // this consumer's tiles: stream numbers congruent to its index
     for (int ti = (wave + kConsumers - base % kConsumers) % kConsumers; ti < nt; ti += kConsumers) {
-      const bool is_new = ti >= n_cache;
-      const int valid = is_new ? 1 : min(kTile, cur.count - ti * kTile);
+      const bool is_new = ti < nt - n_cache;  // the new token comes first
+      const int valid = is_new ? 1 : min(kTile, cur.count - (ti - (nt - n_cache)) * kTile);
       if (valid == kTile) {
         if (!consume_tile(base + ti, valid, false, std::true_type{})) return;
       } else {
@@ -926,7 +1000,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   JPT_TR(if (p.trace && lane == 0) {
     unsigned long long* o = p.trace + (static_cast<size_t>(blockIdx.x) * kWaves + hw_wave) * 8;
     o[0] = tr_tiles; o[1] = tr_wait; o[2] = tr_fold; o[3] = __builtin_amdgcn_s_memrealtime() - tr_start;
-    o[4] = tr_start; o[5] = seq; o[6] = tr_first; o[7] = (__builtin_amdgcn_s_getreg(0xF804) >> 4) & 3;
+    o[4] = tr_start; o[5] = seq; o[6] = tr_first; o[7] = tr_qwait;
   })
 }
 

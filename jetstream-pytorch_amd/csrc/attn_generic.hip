@@ -195,6 +195,12 @@ int32_t check_attn_args(const jpt_attn_args& a, AttnMode mode) {
                 "the new token carries scales exactly when the cache does");
     JPT_REQUIRE(a.q_rows == 1, "the fused new-token term needs q_rows == 1");
   }
+  JPT_REQUIRE((a.new_k_raw == nullptr) == (a.new_v_raw == nullptr), "new_k_raw and new_v_raw go together");
+  if (a.new_k_raw) {
+    JPT_REQUIRE(a.kv_dtype == JPT_I8 && a.k_scale != nullptr, "new_k_raw is for an int8 cache with scales");
+    JPT_REQUIRE(a.new_k && a.new_k_scale && a.new_v_scale, "new_k_raw needs new_k/new_v/new_k_scale/new_v_scale to write to");
+    JPT_REQUIRE(a.new_rounding == JPT_ROUND_TRUNC || a.new_rounding == JPT_ROUND_RNE, "bad new_rounding");
+  }
   if (a.mask) JPT_REQUIRE(a.mask_dtype == JPT_BF16 || a.mask_dtype == JPT_F32, "mask_dtype must be bf16 or f32");
   if (mode == kPaged) {
     JPT_REQUIRE(a.page_table && a.lengths, "paged attention needs page_table and lengths");

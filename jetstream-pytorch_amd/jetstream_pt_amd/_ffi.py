@@ -84,6 +84,7 @@ class AttnArgs(_c.Structure):
       ("max_pages", _i32), ("q_dtype", _i32), ("kv_dtype", _i32),
       ("scale_dtype", _i32), ("scale_heads", _i32), ("mask_dtype", _i32),
       ("sm_scale", _f32), ("force_generic", _i32), ("reuse_plan", _i32),
+      ("new_k_raw", _vp), ("new_v_raw", _vp), ("new_rounding", _i32),
   ]
 
 

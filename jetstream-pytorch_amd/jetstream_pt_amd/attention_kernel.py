@@ -14,6 +14,10 @@ Additions, all keyword-only or optional:
     attended as one more position inside the same launch, which is what the
     reference's lazy-update path does with a second flash_attention call and a
     log-sum-exp merge (layers.py:534-550).
+  * `new_key_raw` / `new_value_raw` on ragged_mha (int8 cache): the step's
+    token before quantisation.  The attention launch then quantises it too
+    (Int8KVCacheGenerate.quantize, cache_manager.py:532-537) and WRITES
+    `new_key` / `new_value` and their scalers, saving the separate launch.
   * `precompute_ragged_block_indices` returns a DecodePlan; pass it where the
     reference passes its `ragged_batch_index` table and every layer of the
     decode step reuses one split plan instead of re-planning per layer.
@@ -24,6 +28,7 @@ import math
 import torch
 
 from . import _ffi
+from .quantize import _rounding_code
 
 
 # ---- workspace and split plans ----------------------------------------------------
@@ -99,7 +104,8 @@ def _scale_tensor(s, paged):
 
 def _attend(mode, xq, keys, values, *, lengths=None, page_table=None, mask=None,
             k_scaler=None, v_scaler=None, sm_scale=None, new_key=None,
-            new_value=None, new_k_scaler=None, new_v_scaler=None, want_stats=False,
+            new_value=None, new_k_scaler=None, new_v_scaler=None, new_key_raw=None,
+            new_value_raw=None, new_rounding="trunc", want_stats=False,
             plan=None, force_generic=False):
   """xq (B, Hq, T, D); keys/values (B, Hkv, S, D) or pages (Hkv, P, ps, D).
   Returns (o (B, Hq, T, D), max (B, Hq, T) | None, denom (B, Hq, T) | None)."""
@@ -169,6 +175,20 @@ def _attend(mode, xq, keys, values, *, lengths=None, page_table=None, mask=None,
       nvs = _ffi.dev(new_v_scaler, "new_v_scaler").to(ks.dtype)
       a.new_k_scale, a.new_v_scale = _ffi.ptr(nks), _ffi.ptr(nvs)
       keep += [nks, nvs]
+    if new_key_raw is not None:
+      # the launch quantises the token itself: new_key/new_value and their
+      # scalers are written, so they must be the caller's own tensors
+      rk, rv = _ffi.dev(new_key_raw, "new_key_raw"), _ffi.dev(new_value_raw, "new_value_raw")
+      if rk.shape != (b, hkv, 1, d) or rk.dtype != torch.bfloat16 or rv.shape != rk.shape \
+          or rv.dtype != rk.dtype or not (rk.is_contiguous() and rv.is_contiguous()):
+        raise ValueError("new_key_raw/new_value_raw must be contiguous bf16 (batch, kv_heads, 1, dim)")
+      if new_k_scaler is None or nks is not new_k_scaler or nvs is not new_v_scaler \
+          or nk is not new_key or nv is not new_value:
+        raise ValueError("with new_key_raw, new_key/new_value and their scalers are outputs: "
+                         "contiguous device tensors in the cache's dtypes")
+      a.new_k_raw, a.new_v_raw = _ffi.ptr(rk), _ffi.ptr(rv)
+      a.new_rounding = _rounding_code(new_rounding)
+      keep += [rk, rv]
   a.sm_scale = 1.0 / math.sqrt(d) if sm_scale is None else float(sm_scale)
   a.force_generic = int(force_generic)
 
@@ -250,7 +270,8 @@ def ragged_mha(q, k, v, layer, start, end, ragged_batch_index=None,
                ragged_block_index=None, k_scaler=None, v_scaler=None, bk=512,
                mask_value=None, normalize_var=True, q_shard_axis=0,
                kv_shard_axis=0, testing=False, *, new_key=None, new_value=None,
-               new_k_scaler=None, new_v_scaler=None):
+               new_k_scaler=None, new_v_scaler=None, new_key_raw=None, new_value_raw=None,
+               new_rounding="trunc"):
   """Left-aligned ragged attention: slot b attends positions < end[b].
 
   Returns what the reference returns: o folded to (B, Hkv, rep*T, D) and
@@ -264,7 +285,8 @@ def ragged_mha(q, k, v, layer, start, end, ragged_batch_index=None,
   out, mx, den = _attend(
       "ragged", q, k, v, lengths=end, k_scaler=k_scaler, v_scaler=v_scaler,
       sm_scale=None if normalize_var else 1.0, new_key=new_key, new_value=new_value,
-      new_k_scaler=new_k_scaler, new_v_scaler=new_v_scaler, want_stats=True, plan=plan)
+      new_k_scaler=new_k_scaler, new_v_scaler=new_v_scaler, new_key_raw=new_key_raw,
+      new_value_raw=new_value_raw, new_rounding=new_rounding, want_stats=True, plan=plan)
   bq, hq, tq, dq = q.shape
   hkv = k.shape[-3]
   rows = hq // hkv * tq

@@ -240,11 +240,18 @@ class Int8KVCacheGenerate:
                                scale_dtype=self.scale_dtype)
     return kq, ks
 
-  def update(self, xk, xv, layer_id: int = 0):
-    """Update kv cache"""
+  def update(self, xk, xv, layer_id: int = 0, *, defer_quantize=False):
+    """Update kv cache.
+
+    defer_quantize (lazy mode only): return the tensors the codes and scales of
+    this token WILL live in without launching the quantiser; the caller hands
+    them to ragged_mha together with xk/xv as new_key_raw/new_value_raw and the
+    attention launch fills them."""
     env = self.env
     b, h, _, d = xk.shape
     dev = xk.device
+    if defer_quantize and not env.lazy_cache_update:
+      raise ValueError("defer_quantize needs lazy_cache_update")
     stash = env.lazy_cache_update and env.new_cache_stacked
     if stash:  # quantise straight into this layer's stash rows
       out = (self.new_ks[layer_id], self.new_vs[layer_id],
@@ -255,7 +262,8 @@ class Int8KVCacheGenerate:
              torch.empty((b, self.scale_heads, 1, 1), dtype=self.scale_dtype, device=dev),
              torch.empty((b, self.scale_heads, 1, 1), dtype=self.scale_dtype, device=dev))
     if env.lazy_cache_update:
-      self._quantize_into(xk, xv, out)
+      if not defer_quantize:
+        self._quantize_into(xk, xv, out)
       if not env.new_cache_stacked:
         if env.generate_cache_stacked:
           self.new_ks.append(out[0])

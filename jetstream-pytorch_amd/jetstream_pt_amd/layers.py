@@ -9,13 +9,17 @@ token attended separately and merged by log-sum-exp.
 With `fuse_new_token` (default) the ragged path hands the new token to the
 attention launch itself, which merges it in its epilogue; the unfused sequence
 (second flash_attention call + lse_merge) stays available and is what the
-other lazy combinations use.  Only this attention part of the reference's
-layers.py is provided; projections, RoPE and norms are outside the KV path.
+other lazy combinations use.  With `fuse_quantize` (default) the int8 kernel
+also leaves the token's quantisation to that launch: cache.update() only names
+the stash rows, and the attention kernel writes codes and scales into them.
+Only this attention part of the reference's layers.py is provided;
+projections, RoPE and norms are outside the KV path.
 """
 
 import torch
 
 from . import attention_kernel as ak
+from .cache_manager import Int8KVCacheGenerate
 
 
 class AttentionKernel:
@@ -87,10 +91,19 @@ class AttentionKernel:
 
 class Int8KVAttentionKernel(AttentionKernel):
 
+  def __init__(self, env, layer_id, *, sm_scale_paged=1.0, fuse_new_token=True, fuse_quantize=True):
+    super().__init__(env, layer_id, sm_scale_paged=sm_scale_paged, fuse_new_token=fuse_new_token)
+    self.fuse_quantize = fuse_quantize and fuse_new_token
+
   def __call__(self, xq, xk, xv, mask, cache, start=None, end=None, ragged_batch_index=None,
                ragged_block_index=None):
     seqlen = xq.shape[2]
-    ret = cache.update(xk, xv, self.layer_id)
+    # the ragged launch can quantise the token itself (one launch less)
+    fuse_quant = (self.fuse_quantize and isinstance(cache, Int8KVCacheGenerate)
+                  and self._will_fuse(seqlen, cache.cache_k) and xk.dtype == torch.bfloat16
+                  and xk.is_contiguous() and xv.is_contiguous())
+    ret = cache.update(xk, xv, self.layer_id, defer_quantize=True) if fuse_quant \
+        else cache.update(xk, xv, self.layer_id)
     if len(ret) == 4:  # int8 pages: (codes k, codes v, scale pages k, scale pages v)
       orig_keys, orig_values, k_scaler, v_scaler = ret
       new_key = new_value = new_k_scaler = new_v_scaler = None
@@ -101,6 +114,8 @@ class Int8KVAttentionKernel(AttentionKernel):
     if new_key is not None and self._will_fuse(seqlen, orig_keys):
       new = dict(new_key=new_key, new_value=new_value, new_k_scaler=new_k_scaler,
                  new_v_scaler=new_v_scaler)
+      if fuse_quant:
+        new.update(new_key_raw=xk, new_value_raw=xv, new_rounding=cache.rounding)
       return self._attend(xq, orig_keys, orig_values, k_scaler, v_scaler, mask, *args,
                           new_token=new)[0]
     existing_output, (existing_max, existing_denom) = self._attend(

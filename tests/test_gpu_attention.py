@@ -211,6 +211,42 @@ def test_fused_new_token_equals_unfused_and_concatenation(quantized):
   check_out(fused.reshape(b, hq, 1, d), wo, "fused vs closed form")
 
 
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (16, 4, 128), (8, 1, 128), (16, 16, 128), (32, 32, 128), (4, 2, 64)])
+@pytest.mark.parametrize("sdt,per_head", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
+@pytest.mark.parametrize("rounding", ["trunc", "rne"])
+def test_attention_launch_quantises_the_new_token(rounding, sdt, per_head, hq, hkv, d):
+  """new_key_raw: the attention launch does the quantiser's work too.  Codes
+  and scales must be the separate quantiser's bit for bit (which the oracle
+  pins), the output that of attending those codes.  32 KV heads and head_dim
+  64 take the library's quantise-first route."""
+  from jetstream_pt_amd import attention_kernel as ak
+  from jetstream_pt_amd.quantize import quantize_kv
+  from oracle import quant as oq
+  g = torch.Generator().manual_seed(311)
+  b, s = 7, 512
+  end = torch.tensor([0, 5, 128, 400, 512, 333, 31], dtype=torch.int32)
+  hs = hkv if per_head else 1
+  q, xk, xv = rnd(g, (b, hq, 1, d)), rnd(g, (b, hkv, 1, d)), rnd(g, (b, hkv, 1, d))
+  xk[2] = 0                      # an all-zero token: scale 0 (trunc) or eps/127 (rne), codes 0
+  xv[3, 0, 0, :5] = 300.0        # a dominant element
+  k, v, ks, vs = int8_cache(g, b, hkv, s, d, hs=hs, sdt=sdt)
+  gq, gk, gv, gks, gvs, gend, gxk, gxv = to_dev(q, k, v, ks, vs, end, xk, xv)
+  wk, wv, wks, wvs = quantize_kv(gxk, gxv, rounding=rounding, scale_heads=hs, scale_dtype=sdt)
+  cdt = None if sdt == torch.bfloat16 else sdt
+  ok_, oks = (oq.quantize_decode if rounding == "trunc" else oq.quantize_insert)(xk, hs, cdt)
+  assert torch.equal(wk.cpu(), ok_) and torch.equal(wks.cpu().reshape(-1), oks.to(sdt).reshape(-1))
+  want, (wm, wl) = ak.ragged_mha(gq, gk, gv, 0, None, gend, None, None, gks, gvs, new_key=wk, new_value=wv,
+                                 new_k_scaler=wks, new_v_scaler=wvs)
+  nk, nv = torch.full_like(wk, 77), torch.full_like(wv, 77)
+  nks, nvs = torch.full_like(wks, -1.0), torch.full_like(wvs, -1.0)
+  got, (m, l) = ak.ragged_mha(gq, gk, gv, 0, None, gend, None, None, gks, gvs, new_key=nk, new_value=nv,
+                              new_k_scaler=nks, new_v_scaler=nvs, new_key_raw=gxk, new_value_raw=gxv,
+                              new_rounding=rounding)
+  assert torch.equal(nk, wk) and torch.equal(nv, wv), "codes"
+  assert torch.equal(nks, wks) and torch.equal(nvs, wvs), "scales"
+  assert torch.equal(got, want) and torch.equal(m, wm) and torch.equal(l, wl)
+
+
 @pytest.mark.parametrize("kind", ["bf16", "int8", "tiny_f32"])
 def test_paged_equals_dense_after_gather(kind):
   from jetstream_pt_amd import attention_kernel as ak
