@@ -514,6 +514,47 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       return true;
     };
 
+    // Issues the loads of one tile into the next ring slot once the slot's
+    // previous tile has been taken, handing over landed tiles meanwhile.  `raw`:
+    // the key/value areas receive the first bytes at tk/tv as they lie (the new
+    // token's unquantised rows) instead of `valid` swizzled rows.
+    auto issue_tile = [&](const char* tk, const char* tv, const char* sc, const float* mk, int valid,
+                          bool raw) -> bool {
+      JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
+      JPT_TR(if (tr_line && issued < 256) tr_line[issued * 8 + 0] = tr_t;)
+      if (!wait_counter(&sm_freed[fill_slot], fill_round, C::kLoadsPerTile)) return false;
+      JPT_TR(if (tr_line && issued < 256) tr_line[issued * 8 + 1] = __builtin_amdgcn_s_memrealtime();)
+      JPT_TR(tr_wait += __builtin_amdgcn_s_memrealtime() - tr_t; if (!tr_first) tr_first = __builtin_amdgcn_s_memrealtime() - tr_start;)
+      char* slot = ring + fill_slot * C::kSlotBytes;
+      JPT_TR(lds_poke(&sm_issue_time[group][fill_slot], static_cast<int>(__builtin_amdgcn_s_memrealtime()));)
+      if (raw) {
+#pragma unroll
+        for (int j = 0; j < kLoadsPerMatrix; ++j) {
+          const uint32_t off = static_cast<uint32_t>(min(64 * j + lane, a.kv_heads * (kD / 8) - 1)) * 16;
+          __builtin_amdgcn_global_load_lds((global_ptr)(tk + off), (lds_ptr)(slot + j * 1024), 16, 0, 0);
+          __builtin_amdgcn_global_load_lds((global_ptr)(tv + off), (lds_ptr)(slot + C::kTileBytes + j * 1024), 16, 0, 0);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < kLoadsPerMatrix; ++j) {
+          const uint32_t off = static_cast<uint32_t>(min(row_of[j], valid - 1)) * C::kRowBytes + piece_off[j];
+          __builtin_amdgcn_global_load_lds((global_ptr)(tk + off), (lds_ptr)(slot + j * 1024), 16, 0, 0);
+          __builtin_amdgcn_global_load_lds((global_ptr)(tv + off), (lds_ptr)(slot + C::kTileBytes + j * 1024), 16, 0, 0);
+        }
+      }
+      char* side = slot + 2 * C::kTileBytes;
+      if (SCALE) {
+        if (lane < 2 * kHalf) __builtin_amdgcn_global_load_lds((global_ptr)sc, (lds_ptr)side, 4, 0, 0);
+      }
+      if (MASK) {
+        if (lane < kTile) __builtin_amdgcn_global_load_lds((global_ptr)(mk + lane), (lds_ptr)(side + 256), 4, 0, 0);
+      }
+      ++issued;
+      loads_issued += C::kLoadsPerTile;
+      if (++fill_slot == C::kSlots) { fill_slot = 0; ++fill_round; }
+      return true;
+    };
+
     int q_seq = 0;  // items with tiles so far: only those have their query rows staged
     for (int k = 0; k < n_rounds; ++k) {
       Item cur;
@@ -538,80 +579,45 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         vt = static_cast<const char*>(a.v) + row0 * C::kRowBytes;
         srow = (static_cast<int64_t>(cur.slot) * a.scale_heads + hs) * a.seq + cur.start;
       }
-      // the step's new token is the item's first tile: the consumer that gets it
-      // has the rest of the item to make up for the extra work it can carry
-      const int n_new = nt - n_cache;
-      for (int ti = 0; ti < nt; ++ti) {
-        const bool is_new = ti < n_new;
-        const int ct = ti - n_new;  // tile of the cache
-        int valid = 1;  // the new token: every row of the tile is that one token
-        const char* sc_src = scale_lane;
-        const char *tk = kt, *tv = vt;
+      // an item's query rows travel ahead of its first tile: loads complete
+      // in order, so they are in LDS when any of its tiles is handed over
+      if (nt > 0 && !issue_q(cur, q_seq++)) return;
+      // The step's new token is the item's first tile: the consumer that gets it
+      // has the rest of the item to make up for the extra work it can carry.
+      if (nt > n_cache) {
+        const int64_t row = static_cast<int64_t>(cur.slot) * a.kv_heads + cur.h;
+        const char* tk = static_cast<const char*>(a.new_k) + row * C::kRowBytes;
+        const char* tv = static_cast<const char*>(a.new_v) + row * C::kRowBytes;
+        if (quant_new) {  // the bf16 rows of all the slot's heads, copied as they lie
+          const int64_t raw = static_cast<int64_t>(cur.slot) * a.kv_heads * (kD * 2);
+          tk = static_cast<const char*>(a.new_k_raw) + raw;
+          tv = static_cast<const char*>(a.new_v_raw) + raw;
+        }
+        // float32 scales of the new token come through the ring like any
+        // tile's; bf16 ones are read by the consumer, and the tile loads the
+        // head of the scale tensors only to keep its load count
+        const char* sc = scale_lane;
+        if (SCALE == kScaleF32) sc = new_scale_lane + (static_cast<int64_t>(cur.slot) * a.scale_heads + hs) * kEs;
+        const float* mk = MASK ? static_cast<const float*>(a.mask) + cur.slot * a.mask_stride_b : nullptr;
+        if (!issue_tile(tk, tv, sc, mk, 1, quant_new)) return;
+      }
+      for (int ct = 0; ct < n_cache; ++ct) {
+        const int t0 = cur.start + ct * kTile;
+        const int valid = min(kTile, cur.start + cur.count - t0);
         int64_t ts = srow;
-        if (is_new) {
-          const int64_t row = static_cast<int64_t>(cur.slot) * a.kv_heads + cur.h;
-          tk = static_cast<const char*>(a.new_k) + row * C::kRowBytes;
-          tv = static_cast<const char*>(a.new_v) + row * C::kRowBytes;
-          if (quant_new) {  // the bf16 rows of all the slot's heads, copied as they lie
-            const int64_t raw = static_cast<int64_t>(cur.slot) * a.kv_heads * (kD * 2);
-            tk = static_cast<const char*>(a.new_k_raw) + raw;
-            tv = static_cast<const char*>(a.new_v_raw) + raw;
-          }
-          // float32 scales of the new token come through the ring like any
-          // tile's; bf16 ones are read by the consumer, and the tile loads the
-          // head of the scale tensors only to keep its load count
-          ts = 0;
-          if (SCALE == kScaleF32) {
-            sc_src = new_scale_lane;
-            ts = static_cast<int64_t>(cur.slot) * a.scale_heads + hs;
-          }
-        } else {
-          const int t0 = cur.start + ct * kTile;
-          valid = min(kTile, cur.start + cur.count - t0);
-          if (PAGED) {  // a tile never straddles a page
-            const int64_t in_pool = static_cast<int64_t>(page) * a.page_size + t0 % a.page_size;
-            const int64_t row0 = static_cast<int64_t>(cur.h) * a.total_pages * a.page_size + in_pool;
-            tk = static_cast<const char*>(a.k) + row0 * C::kRowBytes;
-            tv = static_cast<const char*>(a.v) + row0 * C::kRowBytes;
-            ts = static_cast<int64_t>(hs) * a.total_pages * a.page_size + in_pool;
-            // page of the next tile, read while this one is issued
-            const int tn = min(t0 + kTile, cur.start + cur.count - 1);
-            page = load_uniform(a.page_table + (static_cast<int64_t>(cur.slot) * a.max_pages + tn / a.page_size));
-          }
+        if (PAGED) {  // a tile never straddles a page
+          const int64_t in_pool = static_cast<int64_t>(page) * a.page_size + t0 % a.page_size;
+          const int64_t row0 = static_cast<int64_t>(cur.h) * a.total_pages * a.page_size + in_pool;
+          kt = static_cast<const char*>(a.k) + row0 * C::kRowBytes;
+          vt = static_cast<const char*>(a.v) + row0 * C::kRowBytes;
+          ts = static_cast<int64_t>(hs) * a.total_pages * a.page_size + in_pool;
+          // page of the next tile, read while this one is issued
+          const int tn = min(t0 + kTile, cur.start + cur.count - 1);
+          page = load_uniform(a.page_table + (static_cast<int64_t>(cur.slot) * a.max_pages + tn / a.page_size));
         }
-        // an item's query rows travel ahead of its first tile: loads complete
-        // in order, so they are in LDS when any of its tiles is handed over
-        if (ti == 0 && !issue_q(cur, q_seq++)) return;
-        // wait for the slot's previous tile to be taken, handing over landed
-        // tiles meanwhile
-        JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
-        JPT_TR(if (tr_line && issued < 256) tr_line[issued * 8 + 0] = tr_t;)
-        if (!wait_counter(&sm_freed[fill_slot], fill_round, C::kLoadsPerTile)) return;
-        JPT_TR(if (tr_line && issued < 256) tr_line[issued * 8 + 1] = __builtin_amdgcn_s_memrealtime();)
-        JPT_TR(tr_wait += __builtin_amdgcn_s_memrealtime() - tr_t; if (!tr_first) tr_first = __builtin_amdgcn_s_memrealtime() - tr_start;)
-        char* slot = ring + fill_slot * C::kSlotBytes;
-        JPT_TR(lds_poke(&sm_issue_time[group][fill_slot], static_cast<int>(__builtin_amdgcn_s_memrealtime()));)
-#pragma unroll
-        for (int j = 0; j < kLoadsPerMatrix; ++j) {
-          uint32_t off = static_cast<uint32_t>(min(row_of[j], valid - 1)) * C::kRowBytes + piece_off[j];
-          if (is_new && quant_new) off = static_cast<uint32_t>(min(64 * j + lane, a.kv_heads * (kD / 8) - 1)) * 16;
-          __builtin_amdgcn_global_load_lds((global_ptr)(tk + off), (lds_ptr)(slot + j * 1024), 16, 0, 0);
-          __builtin_amdgcn_global_load_lds((global_ptr)(tv + off), (lds_ptr)(slot + C::kTileBytes + j * 1024), 16, 0, 0);
-        }
-        char* side = slot + 2 * C::kTileBytes;
-        if (SCALE) {
-          if (lane < 2 * kHalf)
-            __builtin_amdgcn_global_load_lds((global_ptr)(sc_src + ts * kEs), (lds_ptr)side, 4, 0, 0);
-        }
-        if (MASK) {
-          const float* src = static_cast<const float*>(a.mask) + cur.slot * a.mask_stride_b + (is_new ? 0 : cur.start + ct * kTile);
-          if (lane < kTile)
-            __builtin_amdgcn_global_load_lds((global_ptr)(src + lane), (lds_ptr)(side + 256), 4, 0, 0);
-        }
-        ++issued;
-        loads_issued += C::kLoadsPerTile;
-        if (++fill_slot == C::kSlots) { fill_slot = 0; ++fill_round; }
-        if (!PAGED && !is_new) {
+        const float* mk = MASK ? static_cast<const float*>(a.mask) + cur.slot * a.mask_stride_b + t0 : nullptr;
+        if (!issue_tile(kt, vt, scale_lane + ts * kEs, mk, valid, false)) return;
+        if (!PAGED) {
           kt += kTile * C::kRowBytes;
           vt += kTile * C::kRowBytes;
           srow += kTile;
