@@ -210,17 +210,25 @@ def build_c1(torch, args):
 
 
 def build_paged(torch, args, int8):
-  """c4 (bf16 pages) / c5 (int8 pages, prompt churn): host page allocation once
-  per decode step, then per layer a paged append and a paged attention."""
+  """c4 (bf16 pages) / c5 (int8 pages, prompt churn): page allocation once per
+  decode step, then per layer a paged append and a paged attention.  By default
+  the allocator, its tables and the per-slot lengths live on the device and a
+  decode step is replayed from one HIP graph (allocation, token indices, all
+  layers, position advance); prompt churn is enqueued between replays.
+  args.host_alloc keeps the allocator on the host as the reference does
+  (lengths pulled every step, tables uploaded), which cannot be captured."""
   import numpy as np
 
   from jetstream_pt_amd import attention_kernel as ak
   from jetstream_pt_amd import cache_manager as cm
+  from jetstream_pt_amd import decode_state
   from jetstream_pt_amd import insert as gins
   from jetstream_pt_amd import layers
   from jetstream_pt_amd.environment import JetEngineEnvironment, JetEngineEnvironmentData
-  from jetstream_pt_amd.page_attention_manager import PageAttentionManager
+  from jetstream_pt_amd.page_attention_manager import DevicePageAttentionManager, PageAttentionManager
 
+  host_alloc = bool(getattr(args, "host_alloc", False))
+  log_on = bool(getattr(args, "log", host_alloc))  # index arrays kept for the parity tests
   if int8:
     nl, batch, hq, hkv, ps, total, max_pages, seed = args.layers or 32, 256, 32, 8, 64, 16384, 64, 5
     lengths = seeded_lengths(torch, batch, 600.0, 16, 4096 - 256, seed).numpy().astype(np.int32)
@@ -230,9 +238,15 @@ def build_paged(torch, args, int8):
   env = JetEngineEnvironment(JetEngineEnvironmentData(
       batch_size=batch, num_layers=nl, paged_attention_total_num_pages=total, paged_attention_page_size=ps))
   rng = np.random.default_rng(seed)
-  pam = PageAttentionManager(batch, total, ps, max_pages, free_list_order=rng.permutation(total).astype(np.int32))
-  for slot in range(batch):
-    pam.reserve_pages_insert(slot, int(lengths[slot]))
+  order = rng.permutation(total).astype(np.int32)
+  if host_alloc:
+    pam = PageAttentionManager(batch, total, ps, max_pages, free_list_order=order)
+    for slot in range(batch):
+      pam.reserve_pages_insert(slot, int(lengths[slot]))
+  else:
+    pam = DevicePageAttentionManager(batch, total, ps, max_pages, device=DEV, free_list_order=order)
+    pam.reserve_pages_insert_many(np.arange(batch, dtype=np.int32), lengths)
+  dlens = torch.from_numpy(lengths.copy()).to(DEV)  # the engine's per-slot lengths, device copy
   e_kv = 1 if int8 else 2
   kdt = torch.int8 if int8 else torch.bfloat16
   pools_k = torch.empty((nl, hkv, total, ps, D), dtype=kdt, device=DEV)
@@ -264,41 +278,72 @@ def build_paged(torch, args, int8):
   state = {"lens": lengths.copy(), "decode_steps": 0, "attended": 0, "pages": 0, "inserted": 0, "log": []}
   churn = 16 if int8 else 0
 
-  def host_step():
-    """What the engine does on the host once per decode step."""
+  def to_dev_async(a):
+    return torch.from_numpy(a).pin_memory().to(DEV, non_blocking=True)
+
+  def before_pass():
+    """What the engine does once per decode step before the layers run: new
+    prompts take over some slots, then (host allocator only) pages for the
+    step are reserved and the tables uploaded.  Also the byte accounting."""
     lens = state["lens"]
     if churn:
-      for slot in rng.choice(batch, churn, replace=False):
-        pam.free_pages_resource(int(slot))
-        n = int(rng.integers(64, 1025))
-        _, ids = pam.reserve_pages_insert(int(slot), n)
-        ids = np.array(ids, dtype=np.int32)
-        gins.insert_prefix_pages_int8_stacked(prompt_k[:, :, :n], prompt_v[:, :, :n], pools_k, pools_v, sk, sv, ids)
-        lens[slot] = n
-        state["inserted"] += n
-        state["log"].append(("insert", int(slot), n, ids))
-    pam.fill_new_pages(lens)
-    idx_host = pam.get_page_token_indices(lens)
-    idx = torch.from_numpy(idx_host).to(DEV)
-    state["log"].append(("decode", lens.copy(), idx_host))
-    lens += 1
-    for c in caches:
-      c.page_token_indices = idx
+      slots = rng.choice(batch, churn, replace=False).astype(np.int32)
+      ns = np.array([int(rng.integers(64, 1025)) for _ in slots], dtype=np.int32)
+      if host_alloc:
+        for slot, n in zip(slots, ns):
+          pam.free_pages_resource(int(slot))
+          _, ids = pam.reserve_pages_insert(int(slot), int(n))
+          ids = np.array(ids, dtype=np.int32)
+          gins.insert_prefix_pages_int8_stacked(prompt_k[:, :, :n], prompt_v[:, :, :n], pools_k, pools_v, sk, sv, ids)
+          state["log"].append(("insert", int(slot), int(n), ids))
+      else:
+        dslots, dns = to_dev_async(slots), to_dev_async(ns)
+        pam.free_pages_resource_many(dslots)
+        pam.reserve_pages_insert_many(dslots, dns)
+        dlens.index_copy_(0, dslots.long(), dns)
+        for slot, n in zip(slots, ns):
+          ids = pam.page_indices[int(slot), : (int(n) + ps - 1) // ps]  # device view: no copy
+          gins.insert_prefix_pages_int8_stacked(prompt_k[:, :, :n], prompt_v[:, :, :n], pools_k, pools_v, sk, sv, ids)
+        if log_on:
+          state["log"].append(("free_many", slots.copy()))
+          state["log"].append(("insert_many", slots.copy(), ns.copy(),
+                               [pam.page_indices[int(s), : (int(n) + ps - 1) // ps].cpu().numpy() for s, n in zip(slots, ns)]))
+      lens[slots] = ns
+      state["inserted"] += int(ns.sum())
+    if host_alloc:
+      pam.fill_new_pages(lens)
+      idx_host = pam.get_page_token_indices(lens)
+      idx = torch.from_numpy(idx_host).to(DEV)
+      state["log"].append(("decode", lens.copy(), idx_host))
+      for c in caches:
+        c.page_token_indices = idx
+    elif log_on:
+      state["log"].append(("decode", lens.copy(), None))
+    lens += (lens > 0)
     state["decode_steps"] += 1
     state["attended"] += int(lens.sum())
     state["pages"] += int(((lens + ps - 1) // ps).sum())
 
   def step(i):
     l = i % nl
-    if l == 0:
-      host_step()
-    return kernels[l](xq, xk, xv, None, caches[l])
+    if l == 0 and not host_alloc:  # allocation and token indices for the step, on the device
+      idx = pam.decode_step(dlens)
+      for c in caches:
+        c.page_token_indices = idx
+      if log_on:  # parity tests only: pulls the index array to the host
+        kind, lens_before, _ = state["log"][-1]
+        state["log"][-1] = (kind, lens_before, idx.to_host())
+    out = kernels[l](xq, xk, xv, None, caches[l])
+    if l == nl - 1 and not host_alloc:
+      decode_state.advance(dlens)
+    return out
 
   def attn_only(i):
     l = i % nl
     lens_d, table = pam.device_tables(DEV)
+    plan = ak.paged_decode_plan(pam, lens_d, batch, hq, hkv, ps, max_pages)  # once per table change, as in step()
     return ak.call_paged_attention(env, xq.squeeze(2), pools_k[l], pools_v[l], lens_d, table,
-                                   k_scaler=sk[l] if int8 else None, v_scaler=sv[l] if int8 else None)
+                                   k_scaler=sk[l] if int8 else None, v_scaler=sv[l] if int8 else None, plan=plan)
 
   def bytes_now():
     """Average algorithmic bytes per layer-step / attention launch over the
@@ -310,10 +355,13 @@ def build_paged(torch, args, int8):
     ins = state["inserted"] / n * (hkv * D * 2 * (2 + 1) + 4 * 2) if int8 else 0   # per layer
     return ab + append + ins, ab
 
+  where = "host page allocation (lengths pulled, tables uploaded)" if host_alloc else \
+      "page allocation, token indices and position advance on the device"
   name = ("C5 paged int8 layer-step: per decode step 16 slots freed and 16 prompts quantised into pages (all "
-          "layers), host page allocation; per layer quantised paged append + paged attention" if int8 else
-          "C4 paged bf16 layer-step: host page allocation per decode step; per layer paged append + paged attention")
-  return dict(step=step, attn_only=attn_only, bytes_now=bytes_now, graph=False, pam=pam, pools=(pools_k, pools_v),
+          f"layers), {where}; per layer quantised paged append + paged attention" if int8 else
+          f"C4 paged bf16 layer-step: {where} once per decode step; per layer paged append + paged attention")
+  return dict(step=step, before_pass=before_pass, attn_only=attn_only, bytes_now=bytes_now, graph=not host_alloc,
+              pam=pam, pools=(pools_k, pools_v), dlens=dlens,
               scale_pages=(sk, sv), caches=caches, state=state, xq=xq, xk=xk, xv=xv, env=env,
               prompts=(prompt_k, prompt_v), initial_lengths=lengths,
               config={"workload": name, "batch": batch, "q_heads": hq, "kv_heads": hkv, "head_dim": D,
@@ -342,11 +390,16 @@ def run_gpu(args):
   nl = w["config"]["layers_rotated"]
   use_graph = w["graph"] and not args.no_graph
 
-  def timed(fn, steps, warmup):
+  def timed(fn, steps, warmup, before=None):
     """fn(i) enqueues step i.  Whole passes over the layers are replayed from
     one captured HIP graph where the workload allows (what a serving loop does
-    with a launch-bound decode step); a remainder of steps runs eagerly."""
-    for i in range(max(warmup, nl)):
+    with a launch-bound decode step); a remainder of steps runs eagerly.
+    before(), when given, is the eager per-pass work ahead of layer 0."""
+    before = before or (lambda: None)
+    warmup = (max(warmup, nl) + nl - 1) // nl * nl  # whole passes
+    for i in range(warmup):
+      if i % nl == 0:
+        before()
       fn(i)
     torch.cuda.synchronize()
     graph = None
@@ -355,6 +408,7 @@ def run_gpu(args):
       with torch.cuda.graph(graph):
         for i in range(nl):
           fn(i)
+      before()
       graph.replay()
       torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -362,15 +416,18 @@ def run_gpu(args):
     done = 0
     if graph is not None:
       for _ in range(steps // nl):
+        before()
         graph.replay()
       done = steps // nl * nl
     for i in range(done, steps):
+      if i % nl == 0:
+        before()
       fn(i)
     stop.record()
     torch.cuda.synchronize()
     return start.elapsed_time(stop) / steps
 
-  ms_per_step = timed(w["step"], args.steps, args.warmup)
+  ms_per_step = timed(w["step"], args.steps, args.warmup, w.get("before_pass"))
   if "bytes_now" in w:
     w["step_bytes"], w["attn_bytes"] = w["bytes_now"]()
   attn_ms = timed(w["attn_only"], args.steps, args.warmup)
@@ -466,6 +523,8 @@ def main():
   ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c3")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   ap.add_argument("--no-graph", action="store_true", help="launch every step from Python")
+  ap.add_argument("--host-alloc", action="store_true",
+                  help="c4/c5: page allocator on the host as in the reference (no graph capture)")
   ap.add_argument("--probe-traffic", action="store_true",
                   help="run a few attention launches and calibration copies for a counter run")
   args = ap.parse_args()

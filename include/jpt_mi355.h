@@ -134,6 +134,15 @@ int32_t jpt_paged_append(void* pages_k, void* pages_v, const void* src_k,
                          int32_t total_pages, int32_t page_size,
                          int32_t row_bytes, void* stream);
 
+/* jpt_paged_append with the column count in device memory: `indices` is
+ * (3, indices_stride), of which the first *n_active_dev columns are valid
+ * (what jpt_dpam_decode_step leaves behind); no host copy of the count. */
+int32_t jpt_paged_append_dev(void* pages_k, void* pages_v, const void* src_k,
+                             const void* src_v, const int32_t* indices,
+                             int32_t indices_stride, const int32_t* n_active_dev,
+                             int32_t batch, int32_t heads, int32_t total_pages,
+                             int32_t page_size, int32_t row_bytes, void* stream);
+
 int32_t jpt_paged_gather(void* dst, const void* pages, const int32_t* page_row,
                          int32_t length, int32_t heads, int32_t total_pages,
                          int32_t page_size, int32_t row_bytes, void* stream);
@@ -154,6 +163,10 @@ typedef struct {
   int32_t n_active;
   int32_t batch, heads, total_pages, page_size, dim;
   int32_t in_dtype, scale_dtype, scale_heads, rounding;
+  /* NULL, or the column count in device memory: then n_active is ignored and
+   * `indices` is (3, indices_stride) with the first *n_active_dev columns valid */
+  const int32_t* n_active_dev;
+  int32_t indices_stride;
 } jpt_paged_quant_append_args;
 
 int32_t jpt_paged_append_quant_i8(const jpt_paged_quant_append_args* args,
@@ -343,6 +356,64 @@ int32_t jpt_pam_free(jpt_pam* pam, int32_t slot);
 /* number of pages on the free list; with out != NULL (capacity total_pages)
  * also copies the list in FIFO order. */
 int32_t jpt_pam_free_count(jpt_pam* pam, int32_t* out);
+
+/* ------------------------------------------------------------------------
+ * Device-resident page allocator: PageAttentionManager with its free list,
+ * page table and lengths in HBM and every method a one-workgroup kernel, so a
+ * paged decode step needs no host round trip (the reference pulls input_pos
+ * to the host every step, engine.py:739-745) and can be captured in a HIP
+ * graph.  Same FIFO order and tables as jpt_pam_* / the reference
+ * (page_attention_manager.py:21-64, :145-177, :214-222), bit for bit.
+ *
+ * The caller owns the device arrays.  Kernels cannot raise: a failed request
+ * is skipped and its bit is set in state[2] (JPT_DPAM_*), where it stays until
+ * jpt_dpam_init; every access stays inside the arrays whatever the inputs.
+ *   state[0] ring head, state[1] free pages, state[2] status bits,
+ *   state[3] n_active of the last jpt_dpam_decode_step.
+ * ---------------------------------------------------------------------- */
+#define JPT_DPAM_NOPAGES 1  /* free list ran out (the reference raises queue.Empty) */
+#define JPT_DPAM_OVERFLOW 2 /* a slot needs more than max_pages pages (IndexError) */
+#define JPT_DPAM_BADARG 4   /* slot out of range or negative length */
+
+typedef struct {
+  int32_t* state;          /* (4) */
+  int32_t* ring;           /* (total_pages) free list, FIFO */
+  int32_t* page_indices;   /* (batch, max_pages); unused entries hold total_pages - 1 */
+  int32_t* lengths;        /* (batch) positions the next paged attention attends */
+  int32_t* n_alloc;        /* (batch) pages each slot was handed */
+  int32_t* update_indices; /* (3, batch): rows page, j * page_size + token, slot of
+                              the active slots; first state[3] columns valid */
+  int32_t batch, total_pages, page_size, max_pages;
+} jpt_dpam;
+
+/* Free list = free_order (device, a permutation of the page ids) or 0, 1, 2...;
+ * tables at their initial values (page_attention_manager.py:29-39). */
+int32_t jpt_dpam_init(const jpt_dpam* pam, const int32_t* free_order, void* stream);
+/* reserve_pages_insert for n_req requests, in order.  slots/seq_lens: device
+ * arrays of n_req entries, or NULL to take the single request (slot, seq_len). */
+int32_t jpt_dpam_reserve_insert(const jpt_dpam* pam, const int32_t* slots,
+                                const int32_t* seq_lens, int32_t n_req,
+                                int32_t slot, int32_t seq_len, void* stream);
+/* free_pages_resource for n_req slots, in order (device array, or NULL and `slot`). */
+int32_t jpt_dpam_free(const jpt_dpam* pam, const int32_t* slots, int32_t n_req,
+                      int32_t slot, void* stream);
+/* fill_new_pages(lens) then get_page_token_indices(lens): lens (batch) device. */
+int32_t jpt_dpam_decode_step(const jpt_dpam* pam, const int32_t* lens, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Decode-state bookkeeping of one generate step on the device
+ * (engine.py:774-817).  update_mask: mask[b, input_pos[b]] = 0, or
+ * mask[:, current_position] = 0 with a ring buffer.  advance: input_pos and
+ * lens become x == 0 ? 0 : x + 1 (ring buffer: x + 1).  The mask update reads
+ * input_pos before it advances.  mask (batch, seq) f32 or bf16, rows
+ * mask_stride elements apart, may be NULL; input_pos, lens (batch) int32, lens
+ * may be NULL.
+ * ---------------------------------------------------------------------- */
+int32_t jpt_decode_advance(void* mask, int32_t mask_dtype, int64_t mask_stride,
+                           int32_t* input_pos, int32_t* lens, int32_t batch,
+                           int32_t seq, int32_t ring_buffer,
+                           int32_t current_position, int32_t update_mask,
+                           int32_t advance, void* stream);
 
 #ifdef __cplusplus
 }

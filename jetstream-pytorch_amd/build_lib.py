@@ -17,7 +17,7 @@ OUT_DIR = os.path.join(HERE, "jetstream_pt_amd")
 LIB = os.path.join(OUT_DIR, "libjpt_mi355.so")
 BUILD = os.path.join(HERE, "build")
 
-SOURCES = ["api.cpp", "pam.cpp", "kv_lines.hip", "prefill_insert.hip", "paged_kv.hip", "attn_generic.hip", "attn_decode.hip",
+SOURCES = ["api.cpp", "pam.cpp", "kv_lines.hip", "prefill_insert.hip", "paged_kv.hip", "device_pages.hip", "attn_generic.hip", "attn_decode.hip",
            "attn_decode_i8.hip", "attn_decode_bf16.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

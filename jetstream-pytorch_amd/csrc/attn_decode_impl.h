@@ -74,6 +74,7 @@ constexpr int kOStride = 140;       // padded LDS row of 128 outputs
 constexpr int kLdsBudget = 160 * 1024 / kGroups - 512;  // per group; one workgroup per compute unit
 constexpr int kSpinLimit = 1 << 18;  // tens of milliseconds
 constexpr int kListedItems = 64;     // a worker's first items, read into LDS at start
+constexpr int kStagedPages = 64;     // page ids of an item kept in LDS (later pages are read one by one)
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -306,6 +307,8 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   __shared__ int sm_abort;
   JPT_TR(__shared__ int sm_issue_time[kGroups][C::kSlots];)
   __shared__ __attribute__((aligned(16))) int sm_items_all[kGroups][kListedItems][8];
+  // page ids of the item being issued and of the next one (paged caches)
+  __shared__ int sm_pages_all[PAGED ? kGroups : 1][2][kStagedPages];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int hw_wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, and known to be
@@ -365,6 +368,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   int* const sm_arrived = sm_arrived_all[group];
   int* const sm_folded = sm_folded_all[group];
   int (*const sm_items)[8] = sm_items_all[group];
+  int (*const sm_pages)[kStagedPages] = sm_pages_all[PAGED ? group : 0];
   if (wave == kConsumers) {
     int entry, h;
     const bool in_range = item_index(lane, &entry, &h);
@@ -458,6 +462,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     int loads_issued = 0;                 // load instructions, all tiles and query rows
     int sig_base = 0;                     // loads issued up to the last signalled tile
     uint64_t carries_q = 0;               // bit t % 64: query rows were loaded just before tile t
+    uint64_t carries_p = 0;               // bit t % 64: a row of page ids was loaded just before tile t
     int fill_slot = 0, fill_round = 0;    // issued % kSlots, issued / kSlots
     int sig_slot = 0, sig_round = 1;      // signalled % kSlots, signalled / kSlots + 1
     // Hands every tile that has landed to the consumers.  Loads complete in
@@ -469,13 +474,15 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       const int out = static_cast<int>((ib & 0xF) | (((ib >> 22) & 0x3) << 4));
       const int done = loads_issued - out;
       while (signalled < issued) {
-        const int need = sig_base + C::kLoadsPerTile + (((carries_q >> (signalled & 63)) & 1) ? q_loads : 0);
+        const int need = sig_base + C::kLoadsPerTile + (((carries_q >> (signalled & 63)) & 1) ? q_loads : 0) +
+                         (PAGED ? static_cast<int>((carries_p >> (signalled & 63)) & 1) : 0);
         if (done < need) break;
         lds_poke(&sm_filled[sig_slot], sig_round);  // every lane stores the same word
         JPT_TR(tr_fold += static_cast<unsigned>(static_cast<int>(__builtin_amdgcn_s_memrealtime()) - lds_peek(&sm_issue_time[group][sig_slot]));)
         JPT_TR(if (tr_line && signalled < 256) tr_line[signalled * 8 + 2] = __builtin_amdgcn_s_memrealtime();)
         sig_base = need;
         carries_q &= ~(1ull << (signalled & 63));
+        if (PAGED) carries_p &= ~(1ull << (signalled & 63));
         ++signalled;
         if (++sig_slot == C::kSlots) { sig_slot = 0; ++sig_round; }
       }
@@ -496,6 +503,35 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         __builtin_amdgcn_s_sleep(1);
       }
     };
+    // Bounded wait until the first `target` loads have landed and `room` more
+    // fit under the counter's limit; false = abort.
+    auto wait_landed = [&](int target, int room) -> bool {
+      for (int spins = 0;; ++spins) {
+        signal_landed();
+        const uint32_t ib = __builtin_amdgcn_s_getreg(0xF807);
+        const int out = static_cast<int>((ib & 0xF) | (((ib >> 22) & 0x3) << 4));
+        if (loads_issued - out >= target && loads_issued - sig_base + room <= 63) return true;
+        if (spins > kSpinLimit || lds_peek_uniform(&sm_abort)) {
+          lds_poke(&sm_abort, 1);
+          __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+          return false;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+    };
+    // Paged caches: the first kStagedPages page ids of an item's positions, one
+    // 4-byte load a lane, into page buffer `buf`.  `with_next_tile`: the load is
+    // counted with the next tile to be issued, like query rows (one such load a
+    // tile at most); otherwise the caller waits for it and retires it itself.
+    auto stage_pages = [&](const Item& it, int buf, bool with_next_tile) {
+      const int idx = min(it.start / a.page_size + lane, a.max_pages - 1);  // stays inside the slot's row
+      const int32_t* src = a.page_table + (static_cast<int64_t>(it.slot) * a.max_pages + idx);
+      __builtin_amdgcn_global_load_lds((global_ptr)src, (lds_ptr)&sm_pages[buf][0], 4, 0, 0);
+      loads_issued += 1;
+      if (with_next_tile) carries_p |= 1ull << (issued & 63);
+    };
+    int staged_round = -1;  // round whose page ids were staged while the round before it was issued
+    int staged_ready = 0;   // loads_issued right after that staging load
     // Query rows of the `seq`-th item that has tiles into their buffer: piece
     // 64j + lane of the item's R contiguous 256-byte rows.
     auto issue_q = [&](const Item& it, int seq) -> bool {
@@ -570,9 +606,24 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       // rows of the item's first position in the key/value and scale tensors
       const char *kt = nullptr, *vt = nullptr;
       int64_t srow = 0;
-      int page = 0;
+      const int first_page = PAGED ? cur.start / a.page_size : 0;
+      int page = 0, page_no = -1;  // page id of page number page_no of the slot
       if (PAGED) {
-        page = load_uniform(a.page_table + (static_cast<int64_t>(cur.slot) * a.max_pages + cur.start / a.page_size));
+        if (n_cache > 0) {
+          // page ids of this item: staged during the previous item, or now
+          if (staged_round != k) {
+            // not staged ahead: load them now and wait.  Once this load has
+            // landed so has every load before it, so every issued tile is
+            // handed over and the load can be retired on the spot.
+            if (!wait_landed(0, 1)) return;
+            stage_pages(cur, k & 1, false);
+            if (!wait_landed(loads_issued, 0)) return;
+            signal_landed();
+            sig_base = loads_issued;
+          } else if (!wait_landed(staged_ready, 0)) {
+            return;
+          }
+        }
       } else {
         const int64_t row0 = (static_cast<int64_t>(cur.slot) * a.kv_heads + cur.h) * a.seq + cur.start;
         kt = static_cast<const char*>(a.k) + row0 * C::kRowBytes;
@@ -582,6 +633,22 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       // an item's query rows travel ahead of its first tile: loads complete
       // in order, so they are in LDS when any of its tiles is handed over
       if (nt > 0 && !issue_q(cur, q_seq++)) return;
+      if (PAGED && k + 1 < n_rounds) {
+        // page ids of the next item, so that they have landed when it starts
+        Item nxt;
+        if (k + 1 < kListedItems) {
+          const i32x4 e0 = lds_peek4(&sm_items[k + 1][0]), e1 = lds_peek4(&sm_items[k + 1][4]);
+          nxt = unpack_item(make_int4(e0[0], e0[1], e0[2], e0[3]), make_int4(e1[0], e1[1], e1[2], e1[3]));
+        } else {
+          nxt = fetch(k + 1);
+        }
+        if (nt > 0 && nxt.valid && nxt.count > 0) {  // nt > 0: a tile of this item follows at once
+          if (!wait_landed(0, 1)) return;
+          stage_pages(nxt, (k + 1) & 1, true);
+          staged_round = k + 1;
+          staged_ready = loads_issued;
+        }
+      }
       // The step's new token is the item's first tile: the consumer that gets it
       // has the rest of the item to make up for the extra work it can carry.
       if (nt > n_cache) {
@@ -606,14 +673,19 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         const int valid = min(kTile, cur.start + cur.count - t0);
         int64_t ts = srow;
         if (PAGED) {  // a tile never straddles a page
+          const int pn = t0 / a.page_size;
+          if (pn != page_no) {
+            page_no = pn;
+            page = pn - first_page < kStagedPages
+                       ? lds_peek_uniform(&sm_pages[k & 1][pn - first_page])
+                       : load_uniform(a.page_table + (static_cast<int64_t>(cur.slot) * a.max_pages + pn));
+            page = min(max(page, 0), a.total_pages - 1);  // whatever the table holds, stay inside the pool
+          }
           const int64_t in_pool = static_cast<int64_t>(page) * a.page_size + t0 % a.page_size;
           const int64_t row0 = static_cast<int64_t>(cur.h) * a.total_pages * a.page_size + in_pool;
           kt = static_cast<const char*>(a.k) + row0 * C::kRowBytes;
           vt = static_cast<const char*>(a.v) + row0 * C::kRowBytes;
           ts = static_cast<int64_t>(hs) * a.total_pages * a.page_size + in_pool;
-          // page of the next tile, read while this one is issued
-          const int tn = min(t0 + kTile, cur.start + cur.count - 1);
-          page = load_uniform(a.page_table + (static_cast<int64_t>(cur.slot) * a.max_pages + tn / a.page_size));
         }
         const float* mk = MASK ? static_cast<const float*>(a.mask) + cur.slot * a.mask_stride_b + t0 : nullptr;
         if (!issue_tile(kt, vt, scale_lane + ts * kEs, mk, valid, false)) return;

@@ -1,0 +1,289 @@
+// Device-resident page allocator and decode-state bookkeeping.
+//
+// PageAttentionManager (jetstream_pt/page_attention_manager.py:21-64, :145-177,
+// :214-222) with the free list, the page table and the lengths in HBM.  Every
+// method is one workgroup of 256 threads: the work is a few hundred integers,
+// and one workgroup keeps the FIFO order of the reference (slots served in
+// ascending order, requests in the order given) without any atomics - a
+// slot's place in the hand-out order is a prefix sum over the slots before it.
+// Kernels cannot raise; a request that cannot be served is skipped and leaves
+// a bit in state[2].  No index read from memory is used before it is checked
+// against the array it addresses.
+#include <algorithm>
+
+#include "common.h"
+
+namespace jpt {
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ void raise(const jpt_dpam& d, int bit) { atomicOr(&d.state[2], bit); }
+
+// Exclusive prefix sum of `x` over the workgroup's threads; *total gets the sum.
+__device__ __forceinline__ int block_exclusive_scan(int x, int* total) {
+  __shared__ int s_wave[kThreads / 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int incl = x;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int y = __shfl_up(incl, off);
+    if (lane >= off) incl += y;
+  }
+  __syncthreads();  // s_wave may still be read from the previous call
+  if (lane == 63) s_wave[wave] = incl;
+  __syncthreads();
+  int before = 0, sum = 0;
+#pragma unroll
+  for (int w = 0; w < kThreads / 64; ++w) {
+    if (w < wave) before += s_wave[w];
+    sum += s_wave[w];
+  }
+  *total = sum;
+  return before + incl - x;
+}
+
+__global__ void __launch_bounds__(kThreads)
+dpam_init_kernel(jpt_dpam d, const int32_t* free_order) {
+  const int64_t tid = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = tid; i < d.total_pages; i += step) d.ring[i] = free_order ? free_order[i] : static_cast<int32_t>(i);
+  const int64_t cells = static_cast<int64_t>(d.batch) * d.max_pages;
+  // the sentinel is the last page id, itself allocatable (:30-35)
+  for (int64_t i = tid; i < cells; i += step) d.page_indices[i] = d.total_pages - 1;
+  for (int64_t i = tid; i < d.batch; i += step) {
+    d.lengths[i] = 0;
+    d.n_alloc[i] = 0;
+  }
+  for (int64_t i = tid; i < 3 * static_cast<int64_t>(d.batch); i += step) d.update_indices[i] = 0;
+  if (tid == 0) {
+    d.state[0] = 0;
+    d.state[1] = d.total_pages;
+    d.state[2] = 0;
+    d.state[3] = 0;
+  }
+}
+
+// reserve_pages_insert (:42-52), requests served one after another.
+__global__ void __launch_bounds__(kThreads)
+dpam_reserve_insert_kernel(jpt_dpam d, const int32_t* slots, const int32_t* seq_lens, int n_req,
+                           int slot_imm, int len_imm) {
+  for (int r = 0; r < n_req; ++r) {
+    const int slot = slots ? slots[r] : slot_imm;
+    const int len = seq_lens ? seq_lens[r] : len_imm;
+    const int head = d.state[0], count = d.state[1];
+    __syncthreads();  // everyone has read the state before thread 0 moves it
+    if (slot < 0 || slot >= d.batch || len < 0) {
+      if (threadIdx.x == 0) raise(d, JPT_DPAM_BADARG);
+      continue;
+    }
+    const int n = (len + d.page_size - 1) / d.page_size;
+    if (n > d.max_pages) {
+      if (threadIdx.x == 0) raise(d, JPT_DPAM_OVERFLOW);
+      continue;
+    }
+    if (n > count) {
+      if (threadIdx.x == 0) raise(d, JPT_DPAM_NOPAGES);
+      continue;
+    }
+    int32_t* row = d.page_indices + static_cast<int64_t>(slot) * d.max_pages;
+    for (int i = threadIdx.x; i < n; i += kThreads) row[i] = d.ring[(head + i) % d.total_pages];
+    if (threadIdx.x == 0) {
+      d.state[0] = (head + n) % d.total_pages;
+      d.state[1] = count - n;
+      d.lengths[slot] = len;
+      d.n_alloc[slot] = n;
+    }
+    __syncthreads();  // the next request sees the moved state
+  }
+}
+
+// free_pages_resource (:214-222): the slot's pages go to the tail of the free
+// list in row order; row back to the sentinel, length to 0.
+__global__ void __launch_bounds__(kThreads)
+dpam_free_kernel(jpt_dpam d, const int32_t* slots, int n_req, int slot_imm) {
+  for (int r = 0; r < n_req; ++r) {
+    const int slot = slots ? slots[r] : slot_imm;
+    const int head = d.state[0], count = d.state[1];
+    __syncthreads();
+    if (slot < 0 || slot >= d.batch) {
+      if (threadIdx.x == 0) raise(d, JPT_DPAM_BADARG);
+      continue;
+    }
+    int32_t* row = d.page_indices + static_cast<int64_t>(slot) * d.max_pages;
+    int n = d.n_alloc[slot];
+    n = min(max(n, 0), min(d.max_pages, d.total_pages - count));  // never more than the ring has room for
+    const int tail = (head + count) % d.total_pages;
+    for (int i = threadIdx.x; i < n; i += kThreads) d.ring[(tail + i) % d.total_pages] = row[i];
+    __syncthreads();  // rows are read before they are reset
+    for (int i = threadIdx.x; i < d.max_pages; i += kThreads) row[i] = d.total_pages - 1;
+    if (threadIdx.x == 0) {
+      d.state[1] = count + n;
+      d.n_alloc[slot] = 0;
+      d.lengths[slot] = 0;
+    }
+    __syncthreads();
+  }
+}
+
+// fill_new_pages (:55-64) followed by get_page_token_indices (:145-177) on the
+// same lens.  A slot whose length sits on a page boundary takes the next free
+// page, slots in ascending order; then every slot with lens != 0 gets a column
+// (page of its new token, j * page_size + token offset, slot) in
+// update_indices, j counting the active slots in ascending order, and
+// lengths = lens + 1 (0 where lens == 0).
+__global__ void __launch_bounds__(kThreads)
+dpam_decode_step_kernel(jpt_dpam d, const int32_t* lens) {
+  const int head = d.state[0], count = d.state[1];
+  const int ps = d.page_size;
+  int popped = 0, active = 0;  // running totals over the slots handled so far
+  for (int base = 0; base < d.batch; base += kThreads) {
+    const int b = base + threadIdx.x;
+    int len = b < d.batch ? lens[b] : 0;
+    if (len < 0) {
+      raise(d, JPT_DPAM_BADARG);
+      len = 0;
+    }
+    const int p = len / ps;  // page that receives the token at position len
+    const bool inside = p < d.max_pages;
+    if (len > 0 && !inside) raise(d, JPT_DPAM_OVERFLOW);
+    const bool wants = len > 0 && len % ps == 0 && inside;
+    int n_wants, n_active;
+    const int rank = popped + block_exclusive_scan(wants ? 1 : 0, &n_wants);
+    const int j = active + block_exclusive_scan(len > 0 ? 1 : 0, &n_active);
+    int32_t* row = d.page_indices + static_cast<int64_t>(b < d.batch ? b : 0) * d.max_pages;
+    int page = d.total_pages - 1;
+    if (len > 0 && inside) page = row[p];
+    if (wants) {
+      if (rank < count) {
+        page = d.ring[(head + rank) % d.total_pages];
+        row[p] = page;
+        d.n_alloc[b] = p + 1;
+      } else {
+        raise(d, JPT_DPAM_NOPAGES);
+      }
+    }
+    if (b < d.batch) {
+      d.lengths[b] = len > 0 ? len + 1 : 0;
+      if (len > 0) {
+        d.update_indices[j] = page;
+        d.update_indices[d.batch + j] = j * ps + len % ps;
+        d.update_indices[2 * d.batch + j] = b;
+      }
+    }
+    popped += n_wants;
+    active += n_active;
+  }
+  if (threadIdx.x == 0) {
+    const int given = min(popped, count);
+    d.state[0] = (head + given) % d.total_pages;
+    d.state[1] = count - given;
+    d.state[3] = active;
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+decode_advance_kernel(T* mask, int64_t mask_stride, int32_t* input_pos, int32_t* lens, int batch, int seq,
+                      int ring_buffer, int current_position, int update_mask, int advance) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= batch) return;
+  const int pos = input_pos[b];
+  if (update_mask && mask) {
+    const int at = ring_buffer ? current_position : pos;
+    if (at >= 0 && at < seq) mask[b * mask_stride + at] = static_cast<T>(0);
+  }
+  if (advance) {
+    // engine.py:800-812: `x + 1 % cache_len` is x + 1
+    input_pos[b] = ring_buffer ? pos + 1 : (pos == 0 ? 0 : pos + 1);
+    if (lens) {
+      const int n = lens[b];
+      lens[b] = ring_buffer ? n + 1 : (n == 0 ? 0 : n + 1);
+    }
+  }
+}
+
+int32_t check_dpam(const jpt_dpam* pam) {
+  JPT_REQUIRE(pam != nullptr, "pam is NULL");
+  JPT_REQUIRE(pam->state && pam->ring && pam->page_indices && pam->lengths && pam->n_alloc && pam->update_indices,
+              "jpt_dpam has a NULL array");
+  JPT_REQUIRE(pam->batch > 0 && pam->total_pages > 0 && pam->page_size > 0 && pam->max_pages > 0,
+              "batch, total_pages, page_size, max_pages must be positive");
+  return JPT_OK;
+}
+
+}  // namespace
+}  // namespace jpt
+
+extern "C" {
+
+int32_t jpt_dpam_init(const jpt_dpam* pam, const int32_t* free_order, void* stream) {
+  using namespace jpt;
+  int32_t st = check_dpam(pam);
+  if (st != JPT_OK) return st;
+  const int64_t most = std::max<int64_t>(pam->total_pages, static_cast<int64_t>(pam->batch) * pam->max_pages);
+  const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((most + kThreads - 1) / kThreads, 1024));
+  hipLaunchKernelGGL(dpam_init_kernel, dim3(blocks), dim3(kThreads), 0, static_cast<hipStream_t>(stream), *pam, free_order);
+  return launch_status("dpam_init_kernel");
+}
+
+int32_t jpt_dpam_reserve_insert(const jpt_dpam* pam, const int32_t* slots, const int32_t* seq_lens,
+                                int32_t n_req, int32_t slot, int32_t seq_len, void* stream) {
+  using namespace jpt;
+  int32_t st = check_dpam(pam);
+  if (st != JPT_OK) return st;
+  JPT_REQUIRE((slots == nullptr) == (seq_lens == nullptr), "slots and seq_lens go together");
+  JPT_REQUIRE(n_req >= 0 && (slots != nullptr || n_req <= 1), "n_req must be 0 or 1 without request arrays");
+  if (n_req == 0) return JPT_OK;
+  if (!slots) {
+    JPT_REQUIRE(slot >= 0 && slot < pam->batch, "slot %d out of range", slot);
+    JPT_REQUIRE(seq_len >= 0, "negative seq_len");
+  }
+  hipLaunchKernelGGL(dpam_reserve_insert_kernel, dim3(1), dim3(kThreads), 0, static_cast<hipStream_t>(stream), *pam,
+                     slots, seq_lens, n_req, slot, seq_len);
+  return launch_status("dpam_reserve_insert_kernel");
+}
+
+int32_t jpt_dpam_free(const jpt_dpam* pam, const int32_t* slots, int32_t n_req, int32_t slot, void* stream) {
+  using namespace jpt;
+  int32_t st = check_dpam(pam);
+  if (st != JPT_OK) return st;
+  JPT_REQUIRE(n_req >= 0 && (slots != nullptr || n_req <= 1), "n_req must be 0 or 1 without a slot array");
+  if (n_req == 0) return JPT_OK;
+  if (!slots) JPT_REQUIRE(slot >= 0 && slot < pam->batch, "slot %d out of range", slot);
+  hipLaunchKernelGGL(dpam_free_kernel, dim3(1), dim3(kThreads), 0, static_cast<hipStream_t>(stream), *pam, slots,
+                     n_req, slot);
+  return launch_status("dpam_free_kernel");
+}
+
+int32_t jpt_dpam_decode_step(const jpt_dpam* pam, const int32_t* lens, void* stream) {
+  using namespace jpt;
+  int32_t st = check_dpam(pam);
+  if (st != JPT_OK) return st;
+  JPT_REQUIRE(lens != nullptr, "lens is NULL");
+  hipLaunchKernelGGL(dpam_decode_step_kernel, dim3(1), dim3(kThreads), 0, static_cast<hipStream_t>(stream), *pam, lens);
+  return launch_status("dpam_decode_step_kernel");
+}
+
+int32_t jpt_decode_advance(void* mask, int32_t mask_dtype, int64_t mask_stride, int32_t* input_pos,
+                           int32_t* lens, int32_t batch, int32_t seq, int32_t ring_buffer,
+                           int32_t current_position, int32_t update_mask, int32_t advance, void* stream) {
+  using namespace jpt;
+  JPT_REQUIRE(input_pos != nullptr, "input_pos is NULL");
+  JPT_REQUIRE(batch > 0 && seq > 0, "batch and seq must be positive");
+  if (mask) {
+    JPT_REQUIRE(mask_dtype == JPT_F32 || mask_dtype == JPT_BF16, "mask_dtype must be f32 or bf16");
+    JPT_REQUIRE(mask_stride >= seq, "mask rows overlap");
+  }
+  const dim3 grid((batch + kThreads - 1) / kThreads);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (mask_dtype == JPT_BF16)
+    hipLaunchKernelGGL(decode_advance_kernel<uint16_t>, grid, dim3(kThreads), 0, s, static_cast<uint16_t*>(mask),
+                       mask_stride, input_pos, lens, batch, seq, ring_buffer, current_position, update_mask, advance);
+  else
+    hipLaunchKernelGGL(decode_advance_kernel<float>, grid, dim3(kThreads), 0, s, static_cast<float*>(mask),
+                       mask_stride, input_pos, lens, batch, seq, ring_buffer, current_position, update_mask, advance);
+  return launch_status("decode_advance_kernel");
+}
+
+}  // extern "C"

@@ -61,9 +61,11 @@ int vector_bytes(const jpt_line_tensor& t) {
 struct QuantParams {
   jpt_quant_append_args a;
   // paged destination (jpt_paged_append_quant_i8): rows are addressed through
-  // `indices` (3, n_active) instead of pos
+  // `indices` (3, stride) instead of pos; its first n_active columns count, or
+  // its first *n_active_dev when that is set
   const int32_t* indices;
-  int32_t n_active, total_pages, page_size;
+  const int32_t* n_active_dev;
+  int32_t stride, total_pages, page_size;
 };
 
 template <bool ROUND_BF16>
@@ -82,7 +84,9 @@ __global__ void __launch_bounds__(256) quant_append_kernel(QuantParams p) {
   const jpt_quant_append_args& a = p.a;
   const bool paged = p.indices != nullptr;
   const int tok = blockIdx.x;
-  const int b = paged ? p.indices[2 * p.n_active + tok] : tok;
+  if (paged && p.n_active_dev && tok >= *p.n_active_dev) return;  // whole workgroup
+  const int b = paged ? p.indices[2 * p.stride + tok] : tok;
+  if (b < 0 || b >= a.batch) return;
   const bool is_v = blockIdx.y == 1;
   const void* src = is_v ? a.new_v : a.new_k;
   int8_t* cache = static_cast<int8_t*>(is_v ? a.cache_v : a.cache_k);
@@ -119,7 +123,7 @@ __global__ void __launch_bounds__(256) quant_append_kernel(QuantParams p) {
   bool write_cache = cache != nullptr;
   if (paged) {
     page = p.indices[tok];
-    at = p.indices[p.n_active + tok] % p.page_size;
+    at = p.indices[p.stride + tok] % p.page_size;
     write_cache = write_cache && page >= 0 && page < p.total_pages;
   } else {
     at = a.pos ? a.pos[a.pos_count == 1 ? 0 : b] : 0;
@@ -161,15 +165,17 @@ __global__ void __launch_bounds__(256) quant_append_kernel(QuantParams p) {
   }
 }
 
-// The same computation for the common shape: bf16 input, four elements a
-// thread kept in registers between the absmax pass and the quantise pass
-// (heads * dim == 4 * blockDim), codes stored four at a time.
-template <bool BF16_MATH>
+// The same computation for the common shapes: bf16 input, heads * dim ==
+// M * 1024; a thread keeps M runs of four elements in registers between the
+// absmax pass and the quantise pass, and stores codes four at a time.
+template <bool BF16_MATH, int M>
 __global__ void __launch_bounds__(256) quant_append_vec_kernel(QuantParams p) {
   const jpt_quant_append_args& a = p.a;
   const bool paged = p.indices != nullptr;
   const int tok = blockIdx.x;
-  const int b = paged ? p.indices[2 * p.n_active + tok] : tok;
+  if (paged && p.n_active_dev && tok >= *p.n_active_dev) return;  // whole workgroup
+  const int b = paged ? p.indices[2 * p.stride + tok] : tok;
+  if (b < 0 || b >= a.batch) return;
   const bool is_v = blockIdx.y == 1;
   const uint16_t* src = static_cast<const uint16_t*>(is_v ? a.new_v : a.new_k);
   int8_t* cache = static_cast<int8_t*>(is_v ? a.cache_v : a.cache_k);
@@ -178,8 +184,6 @@ __global__ void __launch_bounds__(256) quant_append_vec_kernel(QuantParams p) {
   void* stash_scale = is_v ? a.out_v_scale : a.out_k_scale;
   const int H = a.heads, D = a.dim, HD = H * D;
   const int groups = a.scale_heads;  // 1 or H
-  const int i0 = 4 * threadIdx.x;    // this thread's elements i0 .. i0 + 3, all of head h
-  const int h = i0 / D, d = i0 - h * D;
   const int64_t src_base = static_cast<int64_t>(b) * HD;
 
   // destination of this token's rows (read early: the loads overlap)
@@ -187,65 +191,86 @@ __global__ void __launch_bounds__(256) quant_append_vec_kernel(QuantParams p) {
   bool write_cache = cache != nullptr;
   if (paged) {
     page = p.indices[tok];
-    at = p.indices[p.n_active + tok] % p.page_size;
+    at = p.indices[p.stride + tok] % p.page_size;
     write_cache = write_cache && page >= 0 && page < p.total_pages;
   } else {
     at = a.pos ? a.pos[a.pos_count == 1 ? 0 : b] : 0;
     write_cache = write_cache && at >= 0 && at < a.seq;
   }
-  const uint2 raw = *reinterpret_cast<const uint2*>(src + src_base + i0);
-  float x[4] = {__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
-                __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u)};
-  float m = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
+  // run c of this thread: elements i0 .. i0 + 3, all of one head
+  float x[M][4], m[M];
+#pragma unroll
+  for (int c = 0; c < M; ++c) {
+    const int i0 = 4 * (threadIdx.x + 256 * c);
+    const uint2 raw = *reinterpret_cast<const uint2*>(src + src_base + i0);
+    x[c][0] = __uint_as_float(raw.x << 16);
+    x[c][1] = __uint_as_float(raw.x & 0xffff0000u);
+    x[c][2] = __uint_as_float(raw.y << 16);
+    x[c][3] = __uint_as_float(raw.y & 0xffff0000u);
+    m[c] = fmaxf(fmaxf(fabsf(x[c][0]), fabsf(x[c][1])), fmaxf(fabsf(x[c][2]), fabsf(x[c][3])));
+  }
 
-  __shared__ float s_red[64];
-  float amax;
+  __shared__ float s_red[4];
+  float amax[M];
   if (groups == 1) {
-    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
-    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = m;
+    float all = m[0];
+#pragma unroll
+    for (int c = 1; c < M; ++c) all = fmaxf(all, m[c]);
+    for (int off = 32; off > 0; off >>= 1) all = fmaxf(all, __shfl_xor(all, off));
+    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = all;
     __syncthreads();
-    amax = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
-  } else {
-    // a head's D / 4 threads are consecutive; D / 4 is a power of two <= 64
-    for (int off = D / 8; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
-    amax = m;
-  }
-  if (a.rounding == JPT_ROUND_RNE) amax = fmaxf(amax, rnd<BF16_MATH>(1e-5f));
-  const float s = rnd<BF16_MATH>(amax / 127.0f);
-
-  int code[4];
-  if (a.rounding == JPT_ROUND_TRUNC) {
+    all = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float q = rnd<BF16_MATH>(x[i] / s);
-      code[i] = (q != q) ? 0 : static_cast<int>(q);  // 0/0 -> 0; cast truncates
-    }
+    for (int c = 0; c < M; ++c) amax[c] = all;
   } else {
-    const float r = rnd<BF16_MATH>(1.0f / s);
+    // a head's D / 4 threads of a run are consecutive; D / 4 is a power of two <= 64
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float q = rnd<BF16_MATH>(x[i] * r);
-      code[i] = static_cast<int>(fminf(fmaxf(rintf(q), -128.f), 127.f));
+    for (int c = 0; c < M; ++c) {
+      for (int off = D / 8; off > 0; off >>= 1) m[c] = fmaxf(m[c], __shfl_xor(m[c], off));
+      amax[c] = m[c];
     }
   }
-  const uint32_t packed = (static_cast<uint32_t>(code[0]) & 0xffu) | ((static_cast<uint32_t>(code[1]) & 0xffu) << 8) |
-                          ((static_cast<uint32_t>(code[2]) & 0xffu) << 16) | (static_cast<uint32_t>(code[3]) << 24);
-  if (stash) *reinterpret_cast<uint32_t*>(stash + src_base + i0) = packed;
-  if (write_cache) {
-    const int64_t row = paged
-        ? (static_cast<int64_t>(h) * p.total_pages + page) * p.page_size + at
-        : (static_cast<int64_t>(b) * H + h) * a.seq + at;
-    *reinterpret_cast<uint32_t*>(cache + row * D + d) = packed;
-  }
-  // one thread per scale group writes the scale
-  if (groups == 1 ? threadIdx.x == 0 : d == 0) {
-    const int g = groups == 1 ? 0 : h;
-    if (stash_scale) store_from_f32(stash_scale, static_cast<int64_t>(b) * groups + g, a.scale_dtype, s);
-    if (write_cache && scale_out) {
-      const int64_t idx = paged
-          ? (static_cast<int64_t>(g) * p.total_pages + page) * p.page_size + at
-          : (static_cast<int64_t>(b) * groups + g) * a.seq + at;
-      store_from_f32(scale_out, idx, a.scale_dtype, s);
+#pragma unroll
+  for (int c = 0; c < M; ++c) {
+    const int i0 = 4 * (threadIdx.x + 256 * c);
+    const int h = i0 / D, d = i0 - h * D;
+    float am = amax[c];
+    if (a.rounding == JPT_ROUND_RNE) am = fmaxf(am, rnd<BF16_MATH>(1e-5f));
+    const float s = rnd<BF16_MATH>(am / 127.0f);
+    int code[4];
+    if (a.rounding == JPT_ROUND_TRUNC) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float q = rnd<BF16_MATH>(x[c][i] / s);
+        code[i] = (q != q) ? 0 : static_cast<int>(q);  // 0/0 -> 0; cast truncates
+      }
+    } else {
+      const float r = rnd<BF16_MATH>(1.0f / s);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float q = rnd<BF16_MATH>(x[c][i] * r);
+        code[i] = static_cast<int>(fminf(fmaxf(rintf(q), -128.f), 127.f));
+      }
+    }
+    const uint32_t packed = (static_cast<uint32_t>(code[0]) & 0xffu) | ((static_cast<uint32_t>(code[1]) & 0xffu) << 8) |
+                            ((static_cast<uint32_t>(code[2]) & 0xffu) << 16) | (static_cast<uint32_t>(code[3]) << 24);
+    if (stash) *reinterpret_cast<uint32_t*>(stash + src_base + i0) = packed;
+    if (write_cache) {
+      const int64_t row = paged
+          ? (static_cast<int64_t>(h) * p.total_pages + page) * p.page_size + at
+          : (static_cast<int64_t>(b) * H + h) * a.seq + at;
+      *reinterpret_cast<uint32_t*>(cache + row * D + d) = packed;
+    }
+    // one thread per scale group writes the scale
+    if (groups == 1 ? (c == 0 && threadIdx.x == 0) : d == 0) {
+      const int g = groups == 1 ? 0 : h;
+      if (stash_scale) store_from_f32(stash_scale, static_cast<int64_t>(b) * groups + g, a.scale_dtype, s);
+      if (write_cache && scale_out) {
+        const int64_t idx = paged
+            ? (static_cast<int64_t>(g) * p.total_pages + page) * p.page_size + at
+            : (static_cast<int64_t>(b) * groups + g) * a.seq + at;
+        store_from_f32(scale_out, idx, a.scale_dtype, s);
+      }
     }
   }
 }
@@ -268,15 +293,21 @@ int32_t launch_quant(const QuantParams& p, int32_t tokens, hipStream_t stream) {
   dim3 grid(tokens, 2);
   const jpt_quant_append_args& a = p.a;
   const int d4 = a.dim / 4;
-  const bool vec = a.in_dtype == JPT_BF16 && a.heads * a.dim == 1024 && a.dim % 4 == 0 &&
+  const int runs = a.heads * a.dim / 1024;  // runs of four elements per thread
+  const bool vec = a.in_dtype == JPT_BF16 && a.heads * a.dim % 1024 == 0 && (runs == 1 || runs == 2 || runs == 4) &&
+                   a.dim % 4 == 0 &&
                    (a.scale_heads == 1 || (d4 <= 64 && (d4 & (d4 - 1)) == 0)) &&
                    aligned(a.new_k, 8) && aligned(a.new_v, 8) && aligned(a.out_k, 4) && aligned(a.out_v, 4) &&
                    aligned(a.cache_k, 4) && aligned(a.cache_v, 4);
   if (vec) {
-    if (a.scale_dtype == JPT_BF16)
-      hipLaunchKernelGGL(quant_append_vec_kernel<true>, grid, dim3(256), 0, stream, p);
-    else
-      hipLaunchKernelGGL(quant_append_vec_kernel<false>, grid, dim3(256), 0, stream, p);
+    const bool bf = a.scale_dtype == JPT_BF16;
+#define JPT_LAUNCH_VEC(M)                                                                          \
+  if (bf) hipLaunchKernelGGL((quant_append_vec_kernel<true, M>), grid, dim3(256), 0, stream, p);   \
+  else hipLaunchKernelGGL((quant_append_vec_kernel<false, M>), grid, dim3(256), 0, stream, p)
+    if (runs == 1) { JPT_LAUNCH_VEC(1); }
+    else if (runs == 2) { JPT_LAUNCH_VEC(2); }
+    else { JPT_LAUNCH_VEC(4); }
+#undef JPT_LAUNCH_VEC
     return launch_status("quant_append_vec_kernel");
   }
   if (p.a.scale_dtype == JPT_BF16)
@@ -348,8 +379,14 @@ int32_t jpt_paged_append_quant_i8(const jpt_paged_quant_append_args* args, void*
   JPT_REQUIRE(args != nullptr, "args is NULL");
   const jpt_paged_quant_append_args& g = *args;
   JPT_REQUIRE(g.new_k && g.new_v && g.pages_k && g.pages_v && g.k_scale_pages && g.v_scale_pages, "NULL tensor argument");
-  JPT_REQUIRE(g.n_active >= 0 && g.n_active <= g.batch, "n_active must be 0..batch");
-  JPT_REQUIRE(g.n_active == 0 || g.indices != nullptr, "indices is NULL");
+  const bool dev_count = g.n_active_dev != nullptr;
+  if (dev_count) {
+    JPT_REQUIRE(g.indices != nullptr && g.indices_stride >= 1 && g.indices_stride <= g.batch,
+                "with n_active_dev, indices must be (3, indices_stride), indices_stride in 1..batch");
+  } else {
+    JPT_REQUIRE(g.n_active >= 0 && g.n_active <= g.batch, "n_active must be 0..batch");
+    JPT_REQUIRE(g.n_active == 0 || g.indices != nullptr, "indices is NULL");
+  }
   JPT_REQUIRE(g.total_pages > 0 && g.page_size > 0, "total_pages and page_size must be positive");
   int32_t st = check_quant_common(g.heads, g.dim, g.in_dtype, g.scale_dtype, g.scale_heads, g.rounding);
   if (st != JPT_OK) return st;
@@ -368,10 +405,11 @@ int32_t jpt_paged_append_quant_i8(const jpt_paged_quant_append_args* args, void*
   p.a.scale_heads = g.scale_heads;
   p.a.rounding = g.rounding;
   p.indices = g.indices;
-  p.n_active = g.n_active;
+  p.n_active_dev = g.n_active_dev;
+  p.stride = dev_count ? g.indices_stride : g.n_active;
   p.total_pages = g.total_pages;
   p.page_size = g.page_size;
-  return launch_quant(p, g.n_active, static_cast<hipStream_t>(stream));
+  return launch_quant(p, dev_count ? g.indices_stride : g.n_active, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -61,15 +61,17 @@ paged_insert_kernel(void* pages_k, void* pages_v, const void* src_k, const void*
   }
 }
 
-// pages[h, page_j, tok_j % ps, :] = src[slot_j, h, 0, :]
+// pages[h, page_j, tok_j % ps, :] = src[slot_j, h, 0, :].  `indices` is
+// (3, stride); the column count is n_active, or *n_active_dev when that is set.
 template <typename V>
 __global__ void __launch_bounds__(256)
 paged_append_kernel(void* pages_k, void* pages_v, const void* src_k, const void* src_v,
-                    const int32_t* indices, int n_active, int batch, int heads,
-                    int total_pages, int page_size, int row_bytes) {
+                    const int32_t* indices, int stride, int n_active, const int32_t* n_active_dev,
+                    int batch, int heads, int total_pages, int page_size, int row_bytes) {
   V* pages = static_cast<V*>(blockIdx.y ? pages_v : pages_k);
   const V* src = static_cast<const V*>(blockIdx.y ? src_v : src_k);
   const int vpr = row_bytes / sizeof(V);
+  if (n_active_dev) n_active = min(max(*n_active_dev, 0), stride);
   const int64_t total = static_cast<int64_t>(n_active) * heads * vpr;
   for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
        i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
@@ -78,9 +80,9 @@ paged_append_kernel(void* pages_k, void* pages_v, const void* src_k, const void*
     const int h = static_cast<int>(r % heads);
     const int j = static_cast<int>(r / heads);
     const int page = indices[j];
-    const int t = indices[n_active + j] % page_size;
-    const int slot = indices[2 * n_active + j];
-    if (page < 0 || page >= total_pages || slot < 0 || slot >= batch) continue;
+    const int t = indices[stride + j] % page_size;
+    const int slot = indices[2 * stride + j];
+    if (page < 0 || page >= total_pages || slot < 0 || slot >= batch || t < 0) continue;
     pages[((static_cast<int64_t>(h) * total_pages + page) * page_size + t) * vpr + v] =
         src[(static_cast<int64_t>(slot) * heads + h) * vpr + v];
   }
@@ -152,7 +154,26 @@ int32_t jpt_paged_append(void* pages_k, void* pages_v, const void* src_k,
   dim3 grid(blocks_for(static_cast<int64_t>(n_active) * heads * (row_bytes / vec)), 2);
   hipStream_t s = static_cast<hipStream_t>(stream);
   JPT_DISPATCH_VEC(vec, paged_append_kernel, grid, s, pages_k, pages_v, src_k, src_v, indices,
-                   n_active, batch, heads, total_pages, page_size, row_bytes);
+                   n_active, n_active, static_cast<const int32_t*>(nullptr), batch, heads, total_pages,
+                   page_size, row_bytes);
+  return launch_status("paged_append_kernel");
+}
+
+int32_t jpt_paged_append_dev(void* pages_k, void* pages_v, const void* src_k,
+                             const void* src_v, const int32_t* indices,
+                             int32_t indices_stride, const int32_t* n_active_dev,
+                             int32_t batch, int32_t heads, int32_t total_pages,
+                             int32_t page_size, int32_t row_bytes, void* stream) {
+  using namespace jpt;
+  JPT_REQUIRE(pages_k && pages_v && src_k && src_v && indices && n_active_dev, "NULL argument");
+  JPT_REQUIRE(batch > 0 && heads > 0 && total_pages > 0 && page_size > 0 && row_bytes > 0, "batch, heads, total_pages, page_size, row_bytes must be positive");
+  JPT_REQUIRE(indices_stride >= 1, "indices_stride must be positive");
+  const int vec = pick_vec(row_bytes, {pages_k, pages_v, src_k, src_v});
+  // sized for every column; blocks past the device-side count find nothing to do
+  dim3 grid(blocks_for(static_cast<int64_t>(indices_stride) * heads * (row_bytes / vec)), 2);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  JPT_DISPATCH_VEC(vec, paged_append_kernel, grid, s, pages_k, pages_v, src_k, src_v, indices,
+                   indices_stride, 0, n_active_dev, batch, heads, total_pages, page_size, row_bytes);
   return launch_status("paged_append_kernel");
 }
 

@@ -54,8 +54,19 @@ class PagedQuantAppendArgs(_c.Structure):
       ("n_active", _i32), ("batch", _i32), ("heads", _i32),
       ("total_pages", _i32), ("page_size", _i32), ("dim", _i32),
       ("in_dtype", _i32), ("scale_dtype", _i32), ("scale_heads", _i32),
-      ("rounding", _i32),
+      ("rounding", _i32), ("n_active_dev", _vp), ("indices_stride", _i32),
   ]
+
+
+class Dpam(_c.Structure):
+  _fields_ = [
+      ("state", _vp), ("ring", _vp), ("page_indices", _vp), ("lengths", _vp),
+      ("n_alloc", _vp), ("update_indices", _vp), ("batch", _i32),
+      ("total_pages", _i32), ("page_size", _i32), ("max_pages", _i32),
+  ]
+
+
+DPAM_NOPAGES, DPAM_OVERFLOW, DPAM_BADARG = 1, 2, 4
 
 
 class PrefillInsertArgs(_c.Structure):
@@ -101,6 +112,7 @@ _sig("jpt_kv_scatter_lines", _i32, _c.POINTER(LineTensor), _i32, _vp, _i32, _i32
 _sig("jpt_kv_append_quant_i8", _i32, _c.POINTER(QuantAppendArgs), _vp)
 _sig("jpt_paged_insert", _i32, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_paged_append", _i32, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp)
+_sig("jpt_paged_append_dev", _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_paged_gather", _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_paged_append_quant_i8", _i32, _c.POINTER(PagedQuantAppendArgs), _vp)
 _sig("jpt_prefill_insert", _i32, _c.POINTER(PrefillInsertArgs), _vp)
@@ -119,6 +131,11 @@ _sig("jpt_pam_fill_new_pages", _i32, _vp, _i32p)
 _sig("jpt_pam_page_token_indices", _i32, _vp, _i32p, _i32p, _i32p)
 _sig("jpt_pam_free", _i32, _vp, _i32)
 _sig("jpt_pam_free_count", _i32, _vp, _i32p)
+_sig("jpt_dpam_init", _i32, _c.POINTER(Dpam), _vp, _vp)
+_sig("jpt_dpam_reserve_insert", _i32, _c.POINTER(Dpam), _vp, _vp, _i32, _i32, _i32, _vp)
+_sig("jpt_dpam_free", _i32, _c.POINTER(Dpam), _vp, _i32, _i32, _vp)
+_sig("jpt_dpam_decode_step", _i32, _c.POINTER(Dpam), _vp, _vp)
+_sig("jpt_decode_advance", _i32, _vp, _i32, _i64, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp)
 
 EXPORTS = (
     "jpt_version", "jpt_last_error", "jpt_kv_scatter_lines",
@@ -128,7 +145,8 @@ EXPORTS = (
     "jpt_attn_paged", "jpt_lse_merge", "jpt_pam_create", "jpt_pam_destroy",
     "jpt_pam_tables", "jpt_pam_reserve_insert", "jpt_pam_reserve_decode",
     "jpt_pam_fill_new_pages", "jpt_pam_page_token_indices", "jpt_pam_free",
-    "jpt_pam_free_count",
+    "jpt_pam_free_count", "jpt_paged_append_dev", "jpt_dpam_init", "jpt_dpam_reserve_insert",
+    "jpt_dpam_free", "jpt_dpam_decode_step", "jpt_decode_advance",
 )
 
 

@@ -46,6 +46,7 @@ class _Workspace:
 
 
 _workspaces = {}
+_dense_workspaces = {}
 
 
 def _shared_workspace(nbytes, device):
@@ -74,7 +75,28 @@ class DecodePlan:
     self.workspace = _Workspace(nbytes, lengths.device)
     args.workspace = _ffi.ptr(self.workspace.buf)
     args.workspace_bytes = nbytes
-    _ffi.check(_ffi.lib.jpt_attn_plan(args, int(self.paged), _ffi.stream()))
+    self._args = args
+    self.replan()
+
+  def replan(self):
+    """Plans again for the current contents of `lengths` (same tensor, same workspace)."""
+    _ffi.check(_ffi.lib.jpt_attn_plan(self._args, int(self.paged), _ffi.stream()))
+
+
+def paged_decode_plan(pam, lengths, batch, q_heads, kv_heads, page_size, max_pages):
+  """The split plan of a paged decode step, planned once per change of the page
+  manager's tables and shared by every layer's call_paged_attention (the paged
+  counterpart of precompute_ragged_block_indices).  Kept on the manager."""
+  key = (batch, q_heads, kv_heads, 1, None, page_size, max_pages)
+  version = getattr(pam, "_version", None)
+  plan = getattr(pam, "_decode_plan", None)
+  if plan is None or plan.key != key or plan.lengths.data_ptr() != lengths.data_ptr():
+    plan = DecodePlan(lengths, batch, q_heads, kv_heads, page_size=page_size, max_pages=max_pages)
+    pam._decode_plan = plan
+  elif version is None or version != pam._decode_plan_version:
+    plan.replan()
+  pam._decode_plan_version = version
+  return plan
 
 
 def precompute_ragged_block_indices(end, batch, q_heads, kv_heads, seq, q_rows=1):
@@ -204,6 +226,20 @@ def _attend(mode, xq, keys, values, *, lengths=None, page_table=None, mask=None,
                                        a.max_pages or None) and lengths is not None \
       and plan.lengths.data_ptr() == lengths.data_ptr():
     ws, a.reuse_plan = plan.workspace, 1
+  elif lengths is None and mode == "dense":
+    # every slot attends all `seq` positions: the split depends on the shape
+    # only, so it is planned once per (stream, shape) into a workspace of its own
+    key = (torch.device(device), torch.cuda.current_stream(device).cuda_stream, b, hq, hkv, t, a.seq)
+    ws = _dense_workspaces.get(key)
+    if ws is None:
+      ws = _Workspace(_ffi.lib.jpt_attn_workspace_bytes(a), device)
+      pa = _ffi.AttnArgs(batch=b, q_heads=hq, kv_heads=hkv, q_rows=t, seq=a.seq,
+                         workspace=_ffi.ptr(ws.buf), workspace_bytes=ws.nbytes)
+      if _ffi.lib.jpt_attn_plan(pa, 0, _ffi.stream()) == _ffi.OK:
+        _dense_workspaces[key] = ws
+        a.reuse_plan = 1
+    else:
+      a.reuse_plan = 1
   else:
     ws = _shared_workspace(_ffi.lib.jpt_attn_workspace_bytes(a), device)
   a.workspace, a.workspace_bytes = _ffi.ptr(ws.buf), ws.nbytes

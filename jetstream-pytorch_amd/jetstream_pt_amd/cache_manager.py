@@ -21,7 +21,7 @@ Keyword-only additions on Int8KVCacheGenerate, defaults reference-literal:
 import torch
 
 from . import _ffi
-from .page_attention_manager import PageAttentionManager
+from .page_attention_manager import DeviceTokenIndices, PageAttentionManager
 from .quantize import _rounding_code
 
 
@@ -352,6 +352,11 @@ class PageKVCacheGenerate:
     key = _ffi.dev(key.to(pk.dtype).contiguous(), "key")
     value = _ffi.dev(value.to(pv.dtype).contiguous(), "value")
     idx = self.page_token_indices
+    if isinstance(idx, DeviceTokenIndices):  # column count stays on the device
+      _ffi.check(_ffi.lib.jpt_paged_append_dev(
+          _ffi.ptr(pk), _ffi.ptr(pv), _ffi.ptr(key), _ffi.ptr(value), _ffi.ptr(idx.indices), idx.stride,
+          _ffi.ptr(idx.n_active), key.shape[0], heads, total, ps, dim * pk.element_size(), _ffi.stream()))
+      return self.cache_k, self.cache_v
     if not (isinstance(idx, torch.Tensor) and idx.is_cuda and idx.dtype == torch.int32):
       idx = _ffi.as_i32(idx, pk.device).reshape(3, -1)
       self.page_token_indices = idx
@@ -401,13 +406,17 @@ class Int8PageKVCacheGenerate:
     heads, total, ps, dim = pk.shape
     key, value = _ffi.dev(key.contiguous(), "key"), _ffi.dev(value.contiguous(), "value")
     idx = self.page_token_indices
-    if not (isinstance(idx, torch.Tensor) and idx.is_cuda and idx.dtype == torch.int32):
+    n_dev, stride = None, 0
+    if isinstance(idx, DeviceTokenIndices):  # column count stays on the device
+      n_dev, stride, idx = idx.n_active, idx.stride, idx.indices
+    elif not (isinstance(idx, torch.Tensor) and idx.is_cuda and idx.dtype == torch.int32):
       idx = _ffi.as_i32(idx, pk.device).reshape(3, -1)
       self.page_token_indices = idx
     idx = idx.contiguous()
     a = _ffi.PagedQuantAppendArgs(
         new_k=_ffi.ptr(key), new_v=_ffi.ptr(value), pages_k=_ffi.ptr(pk), pages_v=_ffi.ptr(pv),
         k_scale_pages=_ffi.ptr(ks), v_scale_pages=_ffi.ptr(vs), indices=_ffi.ptr(idx),
+        n_active_dev=_ffi.ptr(n_dev), indices_stride=stride,
         n_active=idx.shape[1], batch=key.shape[0], heads=heads, total_pages=total, page_size=ps,
         dim=dim, in_dtype=_ffi.dtype_code(key.dtype), scale_dtype=_ffi.dtype_code(ks.dtype),
         scale_heads=ks.shape[0], rounding=_rounding_code(self.rounding))

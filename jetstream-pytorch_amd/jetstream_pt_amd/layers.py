@@ -52,9 +52,12 @@ class AttentionKernel:
     elif env.page_attention and seqlen == 1 and hasattr(cache, "page_attention_manager"):
       pam = cache.page_attention_manager
       lengths, page_indices = pam.device_tables(xq.device)
+      # one split plan per decode step, shared by the layers
+      plan = ak.paged_decode_plan(pam, lengths, bsz, num_heads, keys.shape[0], keys.shape[2],
+                                  page_indices.shape[1])
       local_output = self.page_attention(
           env, torch.squeeze(xq, 2), keys, values, lengths, page_indices,
-          sm_scale=self.sm_scale_paged, k_scaler=k_scaler, v_scaler=v_scaler)
+          sm_scale=self.sm_scale_paged, k_scaler=k_scaler, v_scaler=v_scaler, plan=plan)
     else:
       local_output = self.dense_attention(
           xq=xq, keys=keys, values=values, k_scaler=k_scaler, v_scaler=v_scaler, mask=local_mask)

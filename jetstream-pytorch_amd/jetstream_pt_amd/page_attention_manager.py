@@ -1,4 +1,4 @@
-"""PageAttentionManager: host page allocator + the kernels that consume its tables.
+"""PageAttentionManager: page allocator + the kernels that consume its tables.
 
 Same constructor and methods as the reference class
 (jetstream_pt/page_attention_manager.py:11-222).  The free list, the page
@@ -6,9 +6,14 @@ table and the lengths live in the C++ allocator of libjpt_mi355.so;
 `page_indices` and `lengths` are numpy views of that memory, so
 `reserve_pages_insert` returns a view of the table row exactly like the
 reference does.  Tensor arguments are torch tensors on the ROCm device.
+
+DevicePageAttentionManager keeps the same state in HBM and runs every method as
+a small kernel: nothing crosses PCIe during a decode step, and the step can be
+captured in a HIP graph.  Same hand-out order and tables as the host class.
 """
 
 import ctypes
+import queue
 from typing import List, Tuple
 
 import numpy as np
@@ -42,7 +47,12 @@ class PageAttentionManager:
     self.page_indices = np.ctypeslib.as_array(pi, shape=(batch_size, max_pages_per_sequence))
     self._lengths = np.ctypeslib.as_array(ln, shape=(batch_size,))
     self._scratch = np.empty(3 * batch_size, dtype=np.int32)
+    self._touch()
+
+  def _touch(self):
+    """The tables changed: device copies and split plans made from them are stale."""
     self._device_tables = None
+    self._version = getattr(self, "_version", 0) + 1
 
   def __del__(self, _destroy=_ffi.lib.jpt_pam_destroy):
     handle, self._handle = getattr(self, "_handle", None), None
@@ -58,7 +68,7 @@ class PageAttentionManager:
     # the reference rebinds `lengths` (page_attention_manager.py:167); here the
     # storage belongs to the allocator, so assignment copies into it
     self._lengths[:] = np.asarray(value, dtype=np.int32)
-    self._device_tables = None
+    self._touch()
 
   @staticmethod
   def _i32(a):
@@ -69,13 +79,13 @@ class PageAttentionManager:
   def reserve_pages_insert(self, slot: int, seq_len: int):
     n = ctypes.c_int32()
     _ffi.check(_ffi.lib.jpt_pam_reserve_insert(self._handle, int(slot), int(seq_len), ctypes.byref(n)))
-    self._device_tables = None
+    self._touch()
     return n.value, self.page_indices[slot, : n.value]
 
   # pylint: disable-next=all
   def reserve_pages_decode(self, slot: int, seq_len: int):
     _ffi.check(_ffi.lib.jpt_pam_reserve_decode(self._handle, int(slot), int(seq_len)))
-    self._device_tables = None
+    self._touch()
 
   # pylint: disable-next=all
   def fill_new_pages(self, lens):
@@ -83,7 +93,7 @@ class PageAttentionManager:
     if arr.size != self.batch_size:
       raise ValueError(f"lens must have {self.batch_size} entries")
     _ffi.check(_ffi.lib.jpt_pam_fill_new_pages(self._handle, p))
-    self._device_tables = None
+    self._touch()
 
   # pylint: disable-next=all
   def get_page_token_indices(self, lens):
@@ -93,13 +103,13 @@ class PageAttentionManager:
     n = ctypes.c_int32()
     out = self._scratch.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
     _ffi.check(_ffi.lib.jpt_pam_page_token_indices(self._handle, p, out, ctypes.byref(n)))
-    self._device_tables = None
+    self._touch()
     return self._scratch[: 3 * n.value].reshape(3, n.value).copy()
 
   # pylint: disable-next=all
   def free_pages_resource(self, slot):
     _ffi.check(_ffi.lib.jpt_pam_free(self._handle, int(slot)))
-    self._device_tables = None
+    self._touch()
     return None
 
   free_pages = free_pages_resource
@@ -161,3 +171,177 @@ class PageAttentionManager:
         _ffi.ptr(out), _ffi.ptr(cache), _ffi.ptr(row), lens, heads, total, ps,
         dim * cache.element_size(), _ffi.stream()))
     return out
+
+
+class DeviceTokenIndices:
+  """What get_page_token_indices returns when the tables live on the device:
+  `indices` (3, stride) int32 with the first `n_active[0]` columns valid,
+  `n_active` a one-element int32 device tensor.  The paged caches' update()
+  takes it where it takes the reference's (3, n_active) array."""
+
+  def __init__(self, indices, n_active):
+    self.indices, self.n_active, self.stride = indices, n_active, indices.shape[1]
+
+  def to_host(self):
+    """(3, n_active) numpy array, as the reference returns it (synchronises)."""
+    n = int(self.n_active.item())
+    return self.indices[:, :n].cpu().numpy()
+
+
+class DevicePageAttentionManager(PageAttentionManager):
+  """PageAttentionManager with free list, page table and lengths on the device.
+
+  Methods enqueue one-workgroup kernels on the current stream and return at
+  once.  Differences a caller sees:
+    * `page_indices` and `lengths` are int32 device tensors (views of the
+      allocator's memory, so `reserve_pages_insert` still returns a view of
+      the table row);
+    * `fill_new_pages(lens)` takes the device tensor of per-slot lengths and
+      also prepares what `get_page_token_indices(lens)` returns, a
+      DeviceTokenIndices;
+    * a kernel cannot raise: a request that cannot be served is skipped and
+      remembered; `check()` (synchronises) raises queue.Empty / IndexError /
+      ValueError for it like the host class does at once.
+  """
+
+  # pylint: disable-next=super-init-not-called
+  def __init__(self, batch_size: int, paged_attention_total_num_pages: int,
+               paged_attention_page_size: int, max_pages_per_sequence: int,
+               *, device="cuda", free_list_order=None):
+    self.batch_size = batch_size
+    self.paged_attention_total_num_pages = paged_attention_total_num_pages
+    self.paged_attention_page_size = paged_attention_page_size
+    self.max_pages_per_sequence = max_pages_per_sequence
+    self._handle = None
+    b, total, mp = batch_size, paged_attention_total_num_pages, max_pages_per_sequence
+    if min(b, total, paged_attention_page_size, mp) <= 0:
+      raise ValueError("batch, total pages, page size and pages per sequence must be positive")
+    sizes = [4, total, b * mp, b, b, 3 * b]
+    offs = [0]
+    for n in sizes:
+      offs.append(offs[-1] + (n + 63) // 64 * 64)  # 256-byte aligned pieces
+    self._mem = torch.zeros(offs[-1], dtype=torch.int32, device=device)
+    piece = lambda i: self._mem[offs[i]: offs[i] + sizes[i]]
+    self._state, self._ring = piece(0), piece(1)
+    self.page_indices = piece(2).view(b, mp)
+    self._lengths, self._n_alloc = piece(3), piece(4)
+    self._update_indices = piece(5).view(3, b)
+    self._c = _ffi.Dpam(
+        state=_ffi.ptr(self._state), ring=_ffi.ptr(self._ring), page_indices=_ffi.ptr(self.page_indices),
+        lengths=_ffi.ptr(self._lengths), n_alloc=_ffi.ptr(self._n_alloc),
+        update_indices=_ffi.ptr(self._update_indices), batch=b, total_pages=total,
+        page_size=paged_attention_page_size, max_pages=mp)
+    order = None
+    if free_list_order is not None:
+      arr = np.ascontiguousarray(np.asarray(free_list_order, dtype=np.int32))
+      if arr.shape != (total,) or not np.array_equal(np.sort(arr), np.arange(total, dtype=np.int32)):
+        raise ValueError("free_list_order must list every page id once")
+      order = torch.from_numpy(arr).to(device)
+    _ffi.check(_ffi.lib.jpt_dpam_init(self._c, _ffi.ptr(order), _ffi.stream()))
+    self._keep = order  # read by the enqueued kernel
+    self._token_indices = DeviceTokenIndices(self._update_indices, self._state[3:4])
+    self._stepped = False
+    self._version = 1  # bumped by every launch that changes `lengths`
+
+  def __del__(self):
+    return
+
+  @property
+  def lengths(self):
+    return self._lengths
+
+  @lengths.setter
+  def lengths(self, value):
+    self._lengths.copy_(torch.as_tensor(value, dtype=torch.int32))
+    self._version += 1
+
+  def _req(self, x):
+    return _ffi.as_i32(x, self._mem.device)
+
+  # pylint: disable-next=all
+  def reserve_pages_insert(self, slot: int, seq_len: int):
+    slot, seq_len = int(slot), int(seq_len)
+    _ffi.check(_ffi.lib.jpt_dpam_reserve_insert(self._c, None, None, 1, slot, seq_len, _ffi.stream()))
+    self._version += 1
+    ps = self.paged_attention_page_size
+    n = (seq_len + ps - 1) // ps
+    return n, self.page_indices[slot, :n]
+
+  def reserve_pages_insert_many(self, slots, seq_lens):
+    """reserve_pages_insert for several slots, in the order given, in one launch;
+    slots and seq_lens may be device tensors (no host copy)."""
+    slots, seq_lens = self._req(slots), self._req(seq_lens)
+    if slots.numel() != seq_lens.numel():
+      raise ValueError("slots and seq_lens differ in length")
+    _ffi.check(_ffi.lib.jpt_dpam_reserve_insert(
+        self._c, _ffi.ptr(slots), _ffi.ptr(seq_lens), slots.numel(), 0, 0, _ffi.stream()))
+    self._keep = (slots, seq_lens)
+    self._version += 1
+
+  # pylint: disable-next=all
+  def reserve_pages_decode(self, slot: int, seq_len: int):
+    raise NotImplementedError("the device allocator serves all slots of a step at once: fill_new_pages(lens)")
+
+  # pylint: disable-next=all
+  def fill_new_pages(self, lens):
+    lens = _ffi.dev(lens, "lens")
+    if lens.dtype != torch.int32 or lens.numel() != self.batch_size:
+      raise ValueError(f"lens must be an int32 device tensor of {self.batch_size} entries")
+    _ffi.check(_ffi.lib.jpt_dpam_decode_step(self._c, _ffi.ptr(lens), _ffi.stream()))
+    self._stepped = True
+    self._version += 1
+
+  # pylint: disable-next=all
+  def get_page_token_indices(self, lens):
+    if not self._stepped:
+      raise RuntimeError("call fill_new_pages(lens) first: on the device both run as one kernel")
+    self._stepped = False
+    return self._token_indices
+
+  def decode_step(self, lens):
+    """fill_new_pages(lens) + get_page_token_indices(lens)."""
+    self.fill_new_pages(lens)
+    return self.get_page_token_indices(lens)
+
+  # pylint: disable-next=all
+  def free_pages_resource(self, slot):
+    _ffi.check(_ffi.lib.jpt_dpam_free(self._c, None, 1, int(slot), _ffi.stream()))
+    self._version += 1
+    return None
+
+  free_pages = free_pages_resource
+
+  def free_pages_resource_many(self, slots):
+    slots = self._req(slots)
+    _ffi.check(_ffi.lib.jpt_dpam_free(self._c, _ffi.ptr(slots), slots.numel(), 0, _ffi.stream()))
+    self._keep = slots
+    self._version += 1
+
+  def status(self):
+    """Failure bits recorded by the kernels so far (synchronises)."""
+    return int(self._state[2].item())
+
+  def check(self):
+    bits = self.status()
+    if bits & _ffi.DPAM_NOPAGES:
+      raise queue.Empty("the device free list ran out of pages")
+    if bits & _ffi.DPAM_OVERFLOW:
+      raise IndexError("a slot needed more pages than max_pages_per_sequence")
+    if bits & _ffi.DPAM_BADARG:
+      raise ValueError("a slot id or length given to the device allocator was out of range")
+
+  def unused_page_ids(self):
+    """The free list in hand-out order (synchronises; for tests and accounting)."""
+    head, count = (int(x) for x in self._state[:2].tolist())
+    ring = self._ring.cpu().numpy()
+    total = self.paged_attention_total_num_pages
+    return ring[(head + np.arange(count)) % total]
+
+  def device_tables(self, device):
+    return self._lengths, self.page_indices
+
+  # pylint: disable-next=all
+  def get_compress_kv_cache(self, decode_caches, slot: int):
+    lens, indices = int(self._lengths[slot].item()), self.page_indices[slot]
+    return [(self._compress_cache(k, lens, indices), self._compress_cache(v, lens, indices))
+            for k, v in decode_caches]

@@ -24,8 +24,12 @@ pytestmark = pytest.mark.gpu
 ATOL, RTOL = 1e-2, 1e-2  # attention outputs (bf16), as the reference's own kernel tests use
 
 
-def args(layers):
-  return argparse.Namespace(layers=layers)
+def args(layers, **more):
+  return argparse.Namespace(layers=layers, **more)
+
+
+def as_np(x):
+  return x.cpu().numpy() if isinstance(x, torch.Tensor) else np.asarray(x)
 
 
 def close(got, want, rtol=RTOL):
@@ -130,13 +134,23 @@ def replay_manager(w, seed, total, ps, max_pages, batch):
       om.free_pages_resource(slot)
       num, view = om.reserve_pages_insert(slot, n)
       assert np.array_equal(np.asarray(view[:num]), ids)
+    elif entry[0] == "free_many":
+      for slot in entry[1]:
+        om.free_pages_resource(int(slot))
+    elif entry[0] == "insert_many":
+      for slot, n, ids in zip(*entry[1:]):
+        num, view = om.reserve_pages_insert(int(slot), int(n))
+        assert np.array_equal(np.asarray(view[:num]), ids)
     else:
       _, lens, idx = entry
       om.fill_new_pages(lens)
       assert np.array_equal(om.get_page_token_indices(lens), idx)
   pam = w["pam"]
-  assert np.array_equal(om.page_indices, pam.page_indices)
-  assert np.array_equal(om.lengths, pam.lengths)
+  assert np.array_equal(om.page_indices, as_np(pam.page_indices))
+  assert np.array_equal(om.lengths, as_np(pam.lengths))
+  assert list(om.unused_pages) == pam.unused_page_ids().tolist()
+  if hasattr(pam, "check"):
+    pam.check()
   return om
 
 
@@ -145,7 +159,7 @@ def paged_attention_subset(w, out, layer, slots, int8):
   pam, ps = w["pam"], pk.shape[2]
   for b in slots:
     n = int(pam.lengths[b])
-    pages = torch.from_numpy(pam.page_indices[b, : (n + ps - 1) // ps].astype(np.int64)).to(pk.device)
+    pages = torch.from_numpy(as_np(pam.page_indices[b, : (n + ps - 1) // ps]).astype(np.int64)).to(pk.device)
     k = pk[:, pages].reshape(pk.shape[0], -1, bench.D)[:, :n].cpu()
     v = pv[:, pages].reshape(pk.shape[0], -1, bench.D)[:, :n].cpu()
     ks = vs = None
@@ -157,12 +171,14 @@ def paged_attention_subset(w, out, layer, slots, int8):
     close(out[b:b + 1], want)
 
 
-def test_c4_paged_bf16_decode_steps():
-  w = bench.build_c4(torch, args(1))
+@pytest.mark.parametrize("host_alloc", [False, True])
+def test_c4_paged_bf16_decode_steps(host_alloc):
+  w = bench.build_c4(torch, args(1, host_alloc=host_alloc, log=True))
   pk, pv = w["pools"][0][0], w["pools"][1][0]
   want_k, want_v = pk.clone(), pv.clone()
   out = None
   for i in range(2):  # two decode steps of the one layer
+    w["before_pass"]()
     out = w["step"](i)
   torch.cuda.synchronize()
   replay_manager(w, 4, 32768, 64, 128, 256)
@@ -175,13 +191,16 @@ def test_c4_paged_bf16_decode_steps():
   paged_attention_subset(w, out, 0, range(0, 256, 11), int8=False)
 
 
-def test_c5_paged_int8_prompt_churn_and_decode_steps():
+@pytest.mark.parametrize("host_alloc", [False, True])
+def test_c5_paged_int8_prompt_churn_and_decode_steps(host_alloc):
   nl = 2
-  w = bench.build_c5(torch, args(nl))
+  w = bench.build_c5(torch, args(nl, host_alloc=host_alloc, log=True))
   pools, scales = w["pools"], w["scale_pages"]
   want = [[t[l].clone() for t in (pools[0], pools[1], scales[0], scales[1])] for l in range(nl)]
   out = None
   for i in range(2 * nl):  # two decode steps over both layers
+    if i % nl == 0:
+      w["before_pass"]()
     o = w["step"](i)
     if i % nl == 0:
       out = o
@@ -193,17 +212,21 @@ def test_c5_paged_int8_prompt_churn_and_decode_steps():
   for entry in w["state"]["log"]:
     for l in range(nl):
       wk, wv, wsk, wsv = want[l]
-      if entry[0] == "insert":
-        _, slot, n, ids = entry
-        pages = torch.from_numpy(ids.astype(np.int64)).to(dev)
-        for src, wc, ws in ((w["prompts"][0], wk, wsk), (w["prompts"][1], wv, wsv)):
-          codes, sc = oquant.quantize_insert(src[l, :, :n].cpu()[None], compute_dtype=torch.float32)
-          padded = torch.zeros((8, len(ids) * 64, bench.D), dtype=torch.int8)
-          padded[:, :n] = codes[0]
-          wc[:, pages] = padded.reshape(8, len(ids), 64, bench.D).to(dev)
-          flat = ws[0, pages].reshape(-1)
-          flat[:n] = sc.reshape(-1).to(dev)
-          ws[0, pages] = flat.reshape(len(ids), 64)
+      if entry[0] == "free_many":
+        continue
+      if entry[0] in ("insert", "insert_many"):
+        prompts = [entry[1:]] if entry[0] == "insert" else zip(*entry[1:])
+        for slot, n, ids in prompts:
+          n = int(n)
+          pages = torch.from_numpy(ids.astype(np.int64)).to(dev)
+          for src, wc, ws in ((w["prompts"][0], wk, wsk), (w["prompts"][1], wv, wsv)):
+            codes, sc = oquant.quantize_insert(src[l, :, :n].cpu()[None], compute_dtype=torch.float32)
+            padded = torch.zeros((8, len(ids) * 64, bench.D), dtype=torch.int8)
+            padded[:, :n] = codes[0]
+            wc[:, pages] = padded.reshape(8, len(ids), 64, bench.D).to(dev)
+            flat = ws[0, pages].reshape(-1)
+            flat[:n] = sc.reshape(-1).to(dev)
+            ws[0, pages] = flat.reshape(len(ids), 64)
       else:
         idx = torch.from_numpy(entry[2]).long().to(dev)
         pages, toks, slots = idx[0], idx[1] % 64, idx[2]

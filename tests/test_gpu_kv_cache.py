@@ -106,13 +106,15 @@ def test_int8_cache_modes(name, flags, variant):
 
 @pytest.mark.parametrize("rounding,ofn", [("trunc", oquant.quantize_decode), ("rne", oquant.quantize_insert)])
 @pytest.mark.parametrize("in_dtype,scale_dtype", [(torch.bfloat16, None), (torch.bfloat16, torch.float32), (torch.float32, None)])
-def test_quantiser_wide_dynamic_range(rounding, ofn, in_dtype, scale_dtype):
-  """256 tokens spanning 1e-6 .. 1e3 in magnitude, 8 heads x 128."""
+@pytest.mark.parametrize("heads", [8, 16, 32, 5])
+def test_quantiser_wide_dynamic_range(heads, rounding, ofn, in_dtype, scale_dtype):
+  """256 tokens spanning 1e-6 .. 1e3 in magnitude, heads x 128 (1024, 2048 and
+  4096 elements a token take the register-resident kernel, 640 the generic one)."""
   from jetstream_pt_amd.quantize import quantize_kv
   g = torch.Generator().manual_seed(102)
-  x = (torch.randn((256, 8, 1, 128), generator=g) * torch.logspace(-6, 3, 256).reshape(-1, 1, 1, 1)).to(in_dtype)
-  y = (torch.randn((256, 8, 1, 128), generator=g) * 3).to(in_dtype)
-  for hs in (1, 8):
+  x = (torch.randn((256, heads, 1, 128), generator=g) * torch.logspace(-6, 3, 256).reshape(-1, 1, 1, 1)).to(in_dtype)
+  y = (torch.randn((256, heads, 1, 128), generator=g) * 3).to(in_dtype)
+  for hs in (1, heads):
     kq, vq, ks, vs = quantize_kv(x.to(DEV), y.to(DEV), rounding=rounding, scale_heads=hs, scale_dtype=scale_dtype)
     for got_c, got_s, src in ((kq, ks, x), (vq, vs, y)):
       wc, ws = ofn(src, hs, scale_dtype)
