@@ -103,9 +103,21 @@ typedef struct {
   int32_t pos_count;
   int32_t batch, heads, seq, dim;
   int32_t in_dtype, scale_dtype, scale_heads, rounding;
+  /* NULL, or rotary factors (batch, dim / 2, 2) float32 = (cos, sin) per slot
+   * and pair, i.e. view_as_real(freqs_cis) of the step: new_k is then taken
+   * UNROTATED and apply_rotary_emb (layers.py:368-379) is applied to it first:
+   * pairs (2i, 2i + 1), re = a*cos - b*sin, im = a*sin + b*cos in float32 with one
+   * rounding per op, result rounded to in_dtype.  new_v is never rotated. */
+  const float* rope;
 } jpt_quant_append_args;
 
 int32_t jpt_kv_append_quant_i8(const jpt_quant_append_args* args, void* stream);
+
+/* apply_rotary_emb (layers.py:368-379) on one tensor: x and out (rows, heads,
+ * dim) in dtype (bf16 or f32), out may equal x; freqs (rows, dim / 2, 2) float32.
+ * The query side of the step (and the key side where no fused append takes it). */
+int32_t jpt_rope(void* out, const void* x, const float* freqs, int32_t rows,
+                 int32_t heads, int32_t dim, int32_t dtype, void* stream);
 
 /* ------------------------------------------------------------------------
  * Paged KV cache.  Pages are (heads, total_pages, page_size, row_bytes).
@@ -167,6 +179,7 @@ typedef struct {
    * `indices` is (3, indices_stride) with the first *n_active_dev columns valid */
   const int32_t* n_active_dev;
   int32_t indices_stride;
+  const float* rope; /* as in jpt_quant_append_args, indexed by slot */
 } jpt_paged_quant_append_args;
 
 int32_t jpt_paged_append_quant_i8(const jpt_paged_quant_append_args* args,
@@ -299,6 +312,9 @@ typedef struct {
   const void* new_k_raw; /* see above; both or neither */
   const void* new_v_raw;
   int32_t new_rounding;  /* JPT_ROUND_* of the fused quantiser */
+  const float* new_k_rope; /* NULL, or rotary factors (batch, dim / 2, 2) as in
+                              jpt_quant_append_args: new_k_raw is unrotated and is
+                              rotated before it is quantised (needs new_k_raw) */
 } jpt_attn_args;
 
 int64_t jpt_attn_workspace_bytes(const jpt_attn_args* args);

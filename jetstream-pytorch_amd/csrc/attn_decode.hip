@@ -323,9 +323,11 @@ static int32_t attn_entry(const jpt_attn_args* args, jpt::AttnMode mode, void* s
     q.scale_dtype = a.scale_dtype;
     q.scale_heads = a.scale_heads;
     q.rounding = a.new_rounding;
+    q.rope = a.new_k_rope;
     st = jpt_kv_append_quant_i8(&q, stream);
     if (st != JPT_OK) return st;
     a.new_k_raw = a.new_v_raw = nullptr;
+    a.new_k_rope = nullptr;
     if (attn_fast_supported(a, mode)) return attn_fast_launch(a, mode, s);
   }
   return attn_generic_launch(a, mode, s);

@@ -741,20 +741,48 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   // only head cur_h is coded, two elements a lane.  Its codes replace row 0 of
   // the area, in tile layout, and go to the stash; the item of head 0 (every
   // item, with per-head scales) stores the scale.
-  auto quantise_new = [&](char* area, int8_t* stash, void* scale_out) -> float {
+  // `rope`: NULL, or the slot's (cos, sin) factors: the rows are rotated pair by
+  // pair first (keys only), rounded to bf16 as the separate rotary op would.
+  auto quantise_new = [&](char* area, int8_t* stash, void* scale_out, const float* rope) -> float {
     constexpr bool kBf16Math = SCALE == kScaleBF16;
     auto rnd = [](float x) { return kBf16Math ? round_to_bf16(x) : x; };
+    auto rotate = [](float& x, float& y, float c, float s) {
+#pragma clang fp contract(off)  // the products are rounded before they are combined
+      const float xc = x * c, ys = y * s, xs = x * s, yc = y * c;
+      const float re = xc - ys;
+      const float im = xs + yc;
+      x = round_to_bf16(re);
+      y = round_to_bf16(im);
+    };
     const uint32_t pair = *reinterpret_cast<const uint32_t*>(area + cur_h * (kD * 2) + lane * 4);
-    const float x0 = __uint_as_float(pair << 16), x1 = __uint_as_float(pair & 0xffff0000u);
+    float x0 = __uint_as_float(pair << 16), x1 = __uint_as_float(pair & 0xffff0000u);
+    if (rope) {  // the lane's elements 2 * lane, 2 * lane + 1 of the head are pair number `lane`
+      const float2 cs = *reinterpret_cast<const float2*>(rope + 2 * lane);
+      rotate(x0, x1, cs.x, cs.y);
+    }
     float m = fmaxf(fabsf(x0), fabsf(x1));
     if (a.scale_heads == 1) {
       for (int at = lane * 32; at < a.kv_heads * (kD * 2); at += 64 * 32) {
         const uint4 r0 = *reinterpret_cast<const uint4*>(area + at);
         const uint4 r1 = *reinterpret_cast<const uint4*>(area + at + 16);
         const uint32_t raw[8] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w};
+        float f[16];
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          m = fmaxf(m, fmaxf(fabsf(__uint_as_float(raw[i] << 16)), fabsf(__uint_as_float(raw[i] & 0xffff0000u))));
+        for (int i = 0; i < 8; ++i) {
+          f[2 * i] = __uint_as_float(raw[i] << 16);
+          f[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
+        }
+        if (rope) {  // byte `at` of the rows is element (at % 256) / 2 of its head: eight pairs from there
+          const float4* cs4 = reinterpret_cast<const float4*>(rope + (at % (kD * 2)) / 2);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float4 cs = cs4[i];
+            rotate(f[4 * i], f[4 * i + 1], cs.x, cs.y);
+            rotate(f[4 * i + 2], f[4 * i + 3], cs.z, cs.w);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) m = fmaxf(m, fabsf(f[i]));
       }
     }
 #pragma unroll
@@ -798,8 +826,9 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     float new_ks = 0.f, new_vs = 0.f;
     const bool quant_here = !FULL && is_new && quant_new;
     if (quant_here) {
-      new_ks = quantise_new(slot, static_cast<int8_t*>(const_cast<void*>(a.new_k)), const_cast<void*>(a.new_k_scale));
-      new_vs = quantise_new(slot + C::kTileBytes, static_cast<int8_t*>(const_cast<void*>(a.new_v)), const_cast<void*>(a.new_v_scale));
+      const float* rope = a.new_k_rope ? a.new_k_rope + static_cast<int64_t>(cur_slot) * kD : nullptr;
+      new_ks = quantise_new(slot, static_cast<int8_t*>(const_cast<void*>(a.new_k)), const_cast<void*>(a.new_k_scale), rope);
+      new_vs = quantise_new(slot + C::kTileBytes, static_cast<int8_t*>(const_cast<void*>(a.new_v)), const_cast<void*>(a.new_v_scale), nullptr);
     }
     T tile;
     tile.read(slot, slot + C::kTileBytes, r, g, pos);

@@ -201,6 +201,8 @@ int32_t check_attn_args(const jpt_attn_args& a, AttnMode mode) {
     JPT_REQUIRE(a.new_k && a.new_k_scale && a.new_v_scale, "new_k_raw needs new_k/new_v/new_k_scale/new_v_scale to write to");
     JPT_REQUIRE(a.new_rounding == JPT_ROUND_TRUNC || a.new_rounding == JPT_ROUND_RNE, "bad new_rounding");
   }
+  JPT_REQUIRE(a.new_k_rope == nullptr || (a.new_k_raw != nullptr && a.dim % 2 == 0 && aligned(a.new_k_rope, 16)),
+              "new_k_rope needs new_k_raw, an even dim and 16-byte aligned factors");
   if (a.mask) JPT_REQUIRE(a.mask_dtype == JPT_BF16 || a.mask_dtype == JPT_F32, "mask_dtype must be bf16 or f32");
   if (mode == kPaged) {
     JPT_REQUIRE(a.page_table && a.lengths, "paged attention needs page_table and lengths");

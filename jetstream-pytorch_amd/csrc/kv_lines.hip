@@ -73,6 +73,17 @@ __device__ __forceinline__ float rnd(float x) {
   return ROUND_BF16 ? round_to_bf16(x) : x;
 }
 
+// One pair of apply_rotary_emb: (a + bi)(c + si), one rounding per op and no
+// fused multiply-add, then rounded to the tensor's dtype.
+__device__ __forceinline__ void rotate_pair(float& a, float& b, float c, float s, bool to_bf16) {
+#pragma clang fp contract(off)  // the products are rounded before they are combined
+  const float ac = a * c, bs = b * s, as = a * s, bc = b * c;
+  const float re = ac - bs;
+  const float im = as + bc;
+  a = to_bf16 ? round_to_bf16(re) : re;
+  b = to_bf16 ? round_to_bf16(im) : im;
+}
+
 // One workgroup per (token, tensor): blockIdx.x = token (slot, or active
 // index j when paged), blockIdx.y = 0 for K, 1 for V.  The op order is the
 // reference's, each op rounded to the scale dtype:
@@ -102,11 +113,21 @@ __global__ void __launch_bounds__(256) quant_append_kernel(QuantParams p) {
   __shared__ float s_red[4];
   __shared__ float s_scale[64 + 1];  // per group (heads <= 64 when per-head)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // element i of the token, rotated when this is the key side and factors are given
+  const float* rope = is_v ? nullptr : a.rope;
+  auto element = [&](int i) -> float {
+    if (!rope) return load_as_f32(src, src_base + i, a.in_dtype);
+    float x0 = load_as_f32(src, src_base + (i & ~1), a.in_dtype);
+    float x1 = load_as_f32(src, src_base + (i | 1), a.in_dtype);
+    const float2 cs = *reinterpret_cast<const float2*>(rope + (static_cast<int64_t>(b) * (D / 2) + (i % D) / 2) * 2);
+    rotate_pair(x0, x1, cs.x, cs.y, a.in_dtype == JPT_BF16);
+    return (i & 1) ? x1 : x0;
+  };
 
   for (int g = 0; g < groups; ++g) {
     float m = 0.f;
     for (int i = threadIdx.x; i < per_group; i += blockDim.x)
-      m = fmaxf(m, fabsf(load_as_f32(src, src_base + g * per_group + i, a.in_dtype)));
+      m = fmaxf(m, fabsf(element(g * per_group + i)));
     for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
     if (lane == 0) s_red[wave] = m;
     __syncthreads();
@@ -133,7 +154,7 @@ __global__ void __launch_bounds__(256) quant_append_kernel(QuantParams p) {
   for (int i = threadIdx.x; i < HD; i += blockDim.x) {
     const int h = i / D, d = i - h * D;
     const float s = s_scale[groups == 1 ? 0 : h];
-    const float x = load_as_f32(src, src_base + i, a.in_dtype);
+    const float x = element(i);
     int code;
     if (a.rounding == JPT_ROUND_TRUNC) {
       const float q = rnd<BF16_MATH>(x / s);
@@ -207,6 +228,12 @@ __global__ void __launch_bounds__(256) quant_append_vec_kernel(QuantParams p) {
     x[c][1] = __uint_as_float(raw.x & 0xffff0000u);
     x[c][2] = __uint_as_float(raw.y << 16);
     x[c][3] = __uint_as_float(raw.y & 0xffff0000u);
+    if (!is_v && a.rope) {  // the run's two pairs: elements d, d + 1 and d + 2, d + 3 of the head
+      const int d = i0 % D;
+      const float4 cs = *reinterpret_cast<const float4*>(a.rope + (static_cast<int64_t>(b) * (D / 2) + d / 2) * 2);
+      rotate_pair(x[c][0], x[c][1], cs.x, cs.y, true);
+      rotate_pair(x[c][2], x[c][3], cs.z, cs.w, true);
+    }
     m[c] = fmaxf(fmaxf(fabsf(x[c][0]), fabsf(x[c][1])), fmaxf(fabsf(x[c][2]), fabsf(x[c][3])));
   }
 
@@ -288,6 +315,23 @@ int32_t check_quant_common(int32_t heads, int32_t dim, int32_t in_dtype,
   return JPT_OK;
 }
 
+// (rows, heads, dim) rotated by (rows, dim / 2, 2); a thread takes one pair
+template <typename T>
+__global__ void __launch_bounds__(256)
+rope_kernel(T* out, const T* x, const float* freqs, int64_t pairs, int heads, int half) {
+  const int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  if (i >= pairs) return;
+  const int64_t row = i / (static_cast<int64_t>(heads) * half);
+  const int p = static_cast<int>(i % half);
+  const float2 cs = *reinterpret_cast<const float2*>(freqs + (row * half + p) * 2);
+  constexpr bool kBf16 = sizeof(T) == 2;
+  float a = kBf16 ? bf16_bits_to_f32(static_cast<uint16_t>(x[2 * i])) : static_cast<float>(x[2 * i]);
+  float b = kBf16 ? bf16_bits_to_f32(static_cast<uint16_t>(x[2 * i + 1])) : static_cast<float>(x[2 * i + 1]);
+  rotate_pair(a, b, cs.x, cs.y, false);
+  out[2 * i] = kBf16 ? static_cast<T>(f32_to_bf16_bits(a)) : static_cast<T>(a);
+  out[2 * i + 1] = kBf16 ? static_cast<T>(f32_to_bf16_bits(b)) : static_cast<T>(b);
+}
+
 int32_t launch_quant(const QuantParams& p, int32_t tokens, hipStream_t stream) {
   if (tokens == 0) return JPT_OK;
   dim3 grid(tokens, 2);
@@ -298,7 +342,7 @@ int32_t launch_quant(const QuantParams& p, int32_t tokens, hipStream_t stream) {
                    a.dim % 4 == 0 &&
                    (a.scale_heads == 1 || (d4 <= 64 && (d4 & (d4 - 1)) == 0)) &&
                    aligned(a.new_k, 8) && aligned(a.new_v, 8) && aligned(a.out_k, 4) && aligned(a.out_v, 4) &&
-                   aligned(a.cache_k, 4) && aligned(a.cache_v, 4);
+                   aligned(a.cache_k, 4) && aligned(a.cache_v, 4) && aligned(a.rope, 16);
   if (vec) {
     const bool bf = a.scale_dtype == JPT_BF16;
 #define JPT_LAUNCH_VEC(M)                                                                          \
@@ -361,6 +405,7 @@ int32_t jpt_kv_append_quant_i8(const jpt_quant_append_args* args, void* stream) 
   JPT_REQUIRE(a.batch > 0, "batch must be positive");
   int32_t st = check_quant_common(a.heads, a.dim, a.in_dtype, a.scale_dtype, a.scale_heads, a.rounding);
   if (st != JPT_OK) return st;
+  JPT_REQUIRE(!a.rope || (a.dim % 2 == 0 && aligned(a.rope, 8)), "rope needs an even dim and 8-byte aligned factors");
   const bool to_cache = a.cache_k != nullptr || a.cache_v != nullptr;
   if (to_cache) {
     JPT_REQUIRE(a.cache_k && a.cache_v && a.k_scale && a.v_scale, "cache_k, cache_v, k_scale, v_scale must all be set");
@@ -372,6 +417,26 @@ int32_t jpt_kv_append_quant_i8(const jpt_quant_append_args* args, void* stream) 
   QuantParams p{};
   p.a = a;
   return launch_quant(p, a.batch, static_cast<hipStream_t>(stream));
+}
+
+int32_t jpt_rope(void* out, const void* x, const float* freqs, int32_t rows, int32_t heads, int32_t dim,
+                 int32_t dtype, void* stream) {
+  using namespace jpt;
+  JPT_REQUIRE(out && x && freqs, "NULL argument");
+  JPT_REQUIRE(rows >= 0 && heads > 0 && dim > 0 && dim % 2 == 0, "rows >= 0, heads > 0 and an even dim are needed");
+  JPT_REQUIRE(dtype == JPT_BF16 || dtype == JPT_F32, "dtype must be bf16 or f32");
+  JPT_REQUIRE(aligned(freqs, 8), "freqs must be 8-byte aligned");
+  const int64_t pairs = static_cast<int64_t>(rows) * heads * (dim / 2);
+  if (pairs == 0) return JPT_OK;
+  const dim3 grid(static_cast<unsigned>((pairs + 255) / 256));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == JPT_BF16)
+    hipLaunchKernelGGL(rope_kernel<uint16_t>, grid, dim3(256), 0, s, static_cast<uint16_t*>(out),
+                       static_cast<const uint16_t*>(x), freqs, pairs, heads, dim / 2);
+  else
+    hipLaunchKernelGGL(rope_kernel<float>, grid, dim3(256), 0, s, static_cast<float*>(out),
+                       static_cast<const float*>(x), freqs, pairs, heads, dim / 2);
+  return launch_status("rope_kernel");
 }
 
 int32_t jpt_paged_append_quant_i8(const jpt_paged_quant_append_args* args, void* stream) {
@@ -388,6 +453,7 @@ int32_t jpt_paged_append_quant_i8(const jpt_paged_quant_append_args* args, void*
     JPT_REQUIRE(g.n_active == 0 || g.indices != nullptr, "indices is NULL");
   }
   JPT_REQUIRE(g.total_pages > 0 && g.page_size > 0, "total_pages and page_size must be positive");
+  JPT_REQUIRE(!g.rope || (g.dim % 2 == 0 && aligned(g.rope, 8)), "rope needs an even dim and 8-byte aligned factors");
   int32_t st = check_quant_common(g.heads, g.dim, g.in_dtype, g.scale_dtype, g.scale_heads, g.rounding);
   if (st != JPT_OK) return st;
   QuantParams p{};
@@ -404,6 +470,7 @@ int32_t jpt_paged_append_quant_i8(const jpt_paged_quant_append_args* args, void*
   p.a.scale_dtype = g.scale_dtype;
   p.a.scale_heads = g.scale_heads;
   p.a.rounding = g.rounding;
+  p.a.rope = g.rope;
   p.indices = g.indices;
   p.n_active_dev = g.n_active_dev;
   p.stride = dev_count ? g.indices_stride : g.n_active;

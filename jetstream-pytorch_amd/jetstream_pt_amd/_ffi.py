@@ -43,7 +43,7 @@ class QuantAppendArgs(_c.Structure):
       ("out_k_scale", _vp), ("out_v_scale", _vp), ("pos", _vp),
       ("pos_count", _i32), ("batch", _i32), ("heads", _i32), ("seq", _i32),
       ("dim", _i32), ("in_dtype", _i32), ("scale_dtype", _i32),
-      ("scale_heads", _i32), ("rounding", _i32),
+      ("scale_heads", _i32), ("rounding", _i32), ("rope", _vp),
   ]
 
 
@@ -55,6 +55,7 @@ class PagedQuantAppendArgs(_c.Structure):
       ("total_pages", _i32), ("page_size", _i32), ("dim", _i32),
       ("in_dtype", _i32), ("scale_dtype", _i32), ("scale_heads", _i32),
       ("rounding", _i32), ("n_active_dev", _vp), ("indices_stride", _i32),
+      ("rope", _vp),
   ]
 
 
@@ -96,6 +97,7 @@ class AttnArgs(_c.Structure):
       ("scale_dtype", _i32), ("scale_heads", _i32), ("mask_dtype", _i32),
       ("sm_scale", _f32), ("force_generic", _i32), ("reuse_plan", _i32),
       ("new_k_raw", _vp), ("new_v_raw", _vp), ("new_rounding", _i32),
+      ("new_k_rope", _vp),
   ]
 
 
@@ -110,6 +112,7 @@ _sig("jpt_version", _i32)
 _sig("jpt_last_error", _c.c_char_p)
 _sig("jpt_kv_scatter_lines", _i32, _c.POINTER(LineTensor), _i32, _vp, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_kv_append_quant_i8", _i32, _c.POINTER(QuantAppendArgs), _vp)
+_sig("jpt_rope", _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_paged_insert", _i32, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_paged_append", _i32, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_paged_append_dev", _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _vp)
@@ -146,7 +149,7 @@ EXPORTS = (
     "jpt_pam_tables", "jpt_pam_reserve_insert", "jpt_pam_reserve_decode",
     "jpt_pam_fill_new_pages", "jpt_pam_page_token_indices", "jpt_pam_free",
     "jpt_pam_free_count", "jpt_paged_append_dev", "jpt_dpam_init", "jpt_dpam_reserve_insert",
-    "jpt_dpam_free", "jpt_dpam_decode_step", "jpt_decode_advance",
+    "jpt_dpam_free", "jpt_dpam_decode_step", "jpt_decode_advance", "jpt_rope",
 )
 
 
@@ -184,6 +187,23 @@ def dev(t, name="tensor"):
   if not t.is_contiguous():
     raise ValueError(f"{name} must be contiguous (shape {tuple(t.shape)}, strides {t.stride()})")
   return t
+
+
+def rope_factors(freqs_cis, rows, dim, name="freqs_cis"):
+  """The step's rotary factors as a contiguous float32 (rows, dim / 2, 2) device
+  tensor of (cos, sin): accepts the reference's complex64 freqs_cis
+  (rows[, 1], dim / 2) - viewed, not copied - or that real layout itself."""
+  f = freqs_cis
+  if not isinstance(f, torch.Tensor) or not f.is_cuda:
+    raise RuntimeError(f"{name} must be a tensor on the ROCm device")
+  if f.is_complex():
+    if f.dtype != torch.complex64:
+      raise ValueError(f"{name} must be complex64")
+    f = torch.view_as_real(f)
+  if f.dtype != torch.float32 or f.numel() != rows * dim or f.shape[-1] != 2:
+    raise ValueError(f"{name} must hold (cos, sin) float32 pairs for {rows} rows of {dim // 2} pairs, "
+                     f"got {tuple(freqs_cis.shape)} {freqs_cis.dtype}")
+  return f.reshape(rows, dim // 2, 2).contiguous()
 
 
 def ptr(t):

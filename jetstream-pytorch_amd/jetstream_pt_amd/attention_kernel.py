@@ -18,6 +18,8 @@ Additions, all keyword-only or optional:
     token before quantisation.  The attention launch then quantises it too
     (Int8KVCacheGenerate.quantize, cache_manager.py:532-537) and WRITES
     `new_key` / `new_value` and their scalers, saving the separate launch.
+    With `new_key_rope` (the step's freqs_cis) the key is taken unrotated and
+    apply_rotary_emb (layers.py:368-379) is applied to it there as well.
   * `precompute_ragged_block_indices` returns a DecodePlan; pass it where the
     reference passes its `ragged_batch_index` table and every layer of the
     decode step reuses one split plan instead of re-planning per layer.
@@ -127,7 +129,7 @@ def _scale_tensor(s, paged):
 def _attend(mode, xq, keys, values, *, lengths=None, page_table=None, mask=None,
             k_scaler=None, v_scaler=None, sm_scale=None, new_key=None,
             new_value=None, new_k_scaler=None, new_v_scaler=None, new_key_raw=None,
-            new_value_raw=None, new_rounding="trunc", want_stats=False,
+            new_value_raw=None, new_rounding="trunc", new_key_rope=None, want_stats=False,
             plan=None, force_generic=False):
   """xq (B, Hq, T, D); keys/values (B, Hkv, S, D) or pages (Hkv, P, ps, D).
   Returns (o (B, Hq, T, D), max (B, Hq, T) | None, denom (B, Hq, T) | None)."""
@@ -211,6 +213,12 @@ def _attend(mode, xq, keys, values, *, lengths=None, page_table=None, mask=None,
       a.new_k_raw, a.new_v_raw = _ffi.ptr(rk), _ffi.ptr(rv)
       a.new_rounding = _rounding_code(new_rounding)
       keep += [rk, rv]
+      if new_key_rope is not None:  # new_key_raw is unrotated
+        rope = _ffi.rope_factors(new_key_rope, b, d, "new_key_rope")
+        a.new_k_rope = _ffi.ptr(rope)
+        keep.append(rope)
+    elif new_key_rope is not None:
+      raise ValueError("new_key_rope goes with new_key_raw (the launch that quantises the token rotates it)")
   a.sm_scale = 1.0 / math.sqrt(d) if sm_scale is None else float(sm_scale)
   a.force_generic = int(force_generic)
 
@@ -307,7 +315,7 @@ def ragged_mha(q, k, v, layer, start, end, ragged_batch_index=None,
                mask_value=None, normalize_var=True, q_shard_axis=0,
                kv_shard_axis=0, testing=False, *, new_key=None, new_value=None,
                new_k_scaler=None, new_v_scaler=None, new_key_raw=None, new_value_raw=None,
-               new_rounding="trunc"):
+               new_rounding="trunc", new_key_rope=None):
   """Left-aligned ragged attention: slot b attends positions < end[b].
 
   Returns what the reference returns: o folded to (B, Hkv, rep*T, D) and
@@ -322,7 +330,8 @@ def ragged_mha(q, k, v, layer, start, end, ragged_batch_index=None,
       "ragged", q, k, v, lengths=end, k_scaler=k_scaler, v_scaler=v_scaler,
       sm_scale=None if normalize_var else 1.0, new_key=new_key, new_value=new_value,
       new_k_scaler=new_k_scaler, new_v_scaler=new_v_scaler, new_key_raw=new_key_raw,
-      new_value_raw=new_value_raw, new_rounding=new_rounding, want_stats=True, plan=plan)
+      new_value_raw=new_value_raw, new_rounding=new_rounding, new_key_rope=new_key_rope,
+      want_stats=True, plan=plan)
   bq, hq, tq, dq = q.shape
   hkv = k.shape[-3]
   rows = hq // hkv * tq

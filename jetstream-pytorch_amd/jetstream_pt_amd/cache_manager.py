@@ -207,7 +207,7 @@ class Int8KVCacheGenerate:
   def _pos(self, count):
     return _ffi.as_i32(self.input_pos, self.cache_k.device, count)
 
-  def _quantize_into(self, xk, xv, out, cache=None, ring=False):
+  def _quantize_into(self, xk, xv, out, cache=None, ring=False, freqs_cis=None):
     """Runs the fused quantiser.  out = (k_codes, v_codes, k_scale, v_scale)
     destinations shaped (B, H, 1, D) / (B, Hs, 1, 1); cache = optional
     (cache_k, cache_v, k_scaler, v_scaler) 4-D views to scatter into."""
@@ -222,6 +222,10 @@ class Int8KVCacheGenerate:
     for t_ in out:
       _ffi.dev(t_, "quantiser output")
     a.out_k, a.out_v, a.out_k_scale, a.out_v_scale = (_ffi.ptr(t_) for t_ in out)
+    rope = None
+    if freqs_cis is not None:  # xk is unrotated: the launch rotates it first
+      rope = _ffi.rope_factors(freqs_cis, b, d)
+      a.rope = _ffi.ptr(rope)
     pos = None
     if cache is not None:
       for t_ in cache:
@@ -240,8 +244,11 @@ class Int8KVCacheGenerate:
                                scale_dtype=self.scale_dtype)
     return kq, ks
 
-  def update(self, xk, xv, layer_id: int = 0, *, defer_quantize=False):
+  def update(self, xk, xv, layer_id: int = 0, *, defer_quantize=False, freqs_cis=None):
     """Update kv cache.
+
+    freqs_cis: the step's rotary factors when xk has NOT been through
+    apply_rotary_emb yet; the quantiser launch then rotates it first.
 
     defer_quantize (lazy mode only): return the tensors the codes and scales of
     this token WILL live in without launching the quantiser; the caller hands
@@ -263,7 +270,7 @@ class Int8KVCacheGenerate:
              torch.empty((b, self.scale_heads, 1, 1), dtype=self.scale_dtype, device=dev))
     if env.lazy_cache_update:
       if not defer_quantize:
-        self._quantize_into(xk, xv, out)
+        self._quantize_into(xk, xv, out, freqs_cis=freqs_cis)
       if not env.new_cache_stacked:
         if env.generate_cache_stacked:
           self.new_ks.append(out[0])
@@ -278,7 +285,7 @@ class Int8KVCacheGenerate:
                  self.k_scaler[layer_id], self.v_scaler[layer_id])
       else:
         cache = (self.cache_k, self.cache_v, self.k_scaler, self.v_scaler)
-      self._quantize_into(xk, xv, out, cache, ring=env.ring_buffer)
+      self._quantize_into(xk, xv, out, cache, ring=env.ring_buffer, freqs_cis=freqs_cis)
     k_quant, v_quant, kscale, vscale = out
     return (self.cache_k, self.cache_v, k_quant, v_quant, self.k_scaler, self.v_scaler,
             kscale, vscale)
@@ -400,7 +407,8 @@ class Int8PageKVCacheGenerate:
     self.stacked = False
     self.rounding = rounding
 
-  def update(self, key, value, layer_id=0):
+  def update(self, key, value, layer_id=0, *, freqs_cis=None):
+    """freqs_cis: rotary factors of the step when `key` is still unrotated."""
     pk, pv = _ffi.dev(self.cache_k, "cache_k"), _ffi.dev(self.cache_v, "cache_v")
     ks, vs = _ffi.dev(self.k_scaler, "k_scale_pages"), _ffi.dev(self.v_scaler, "v_scale_pages")
     heads, total, ps, dim = pk.shape
@@ -420,7 +428,12 @@ class Int8PageKVCacheGenerate:
         n_active=idx.shape[1], batch=key.shape[0], heads=heads, total_pages=total, page_size=ps,
         dim=dim, in_dtype=_ffi.dtype_code(key.dtype), scale_dtype=_ffi.dtype_code(ks.dtype),
         scale_heads=ks.shape[0], rounding=_rounding_code(self.rounding))
+    rope = None
+    if freqs_cis is not None:
+      rope = _ffi.rope_factors(freqs_cis, key.shape[0], dim)
+      a.rope = _ffi.ptr(rope)
     _ffi.check(_ffi.lib.jpt_paged_append_quant_i8(a, _ffi.stream()))
+    del rope
     return self.cache_k, self.cache_v, self.k_scaler, self.v_scaler
 
   def state(self):

@@ -18,8 +18,29 @@ projections, RoPE and norms are outside the KV path.
 
 import torch
 
+from . import _ffi
 from . import attention_kernel as ak
 from .cache_manager import Int8KVCacheGenerate
+
+
+def apply_rotary_emb(xq, xk, freqs_cis):
+  """The reference's apply_rotary_emb (jetstream_pt/layers.py:368-379) as one small
+  launch per tensor: xq, xk (bs, seqlen, heads, dim), freqs_cis (bs, seqlen,
+  dim / 2) complex64.  Either tensor may be None (e.g. xk, when the KV append
+  rotates the key itself); returns (xq_out, xk_out)."""
+  outs = []
+  for x in (xq, xk):
+    if x is None:
+      outs.append(None)
+      continue
+    x = _ffi.dev(x.contiguous(), "x")
+    bs, seqlen, heads, dim = x.shape
+    f = _ffi.rope_factors(freqs_cis, bs * seqlen, dim)
+    out = torch.empty_like(x)
+    _ffi.check(_ffi.lib.jpt_rope(_ffi.ptr(out), _ffi.ptr(x), _ffi.ptr(f), bs * seqlen, heads, dim,
+                                 _ffi.dtype_code(x.dtype), _ffi.stream()))
+    outs.append(out)
+  return tuple(outs)
 
 
 class AttentionKernel:
@@ -99,14 +120,22 @@ class Int8KVAttentionKernel(AttentionKernel):
     self.fuse_quantize = fuse_quantize and fuse_new_token
 
   def __call__(self, xq, xk, xv, mask, cache, start=None, end=None, ragged_batch_index=None,
-               ragged_block_index=None):
+               ragged_block_index=None, *, freqs_cis=None):
+    """freqs_cis (keyword, optional): the step's rotary factors when xk has NOT been
+    through apply_rotary_emb; the launch that quantises the key rotates it first
+    (xq must come rotated).  One token per slot only."""
     seqlen = xq.shape[2]
+    if freqs_cis is not None and (xk.shape[2] != 1 or not hasattr(cache, "rounding")):
+      # no quantiser launch to fold the rotation into: rotate here
+      xk = apply_rotary_emb(None, xk.transpose(1, 2), freqs_cis)[1].transpose(1, 2)
+      freqs_cis = None
+    rope_kw = {} if freqs_cis is None else {"freqs_cis": freqs_cis}
     # the ragged launch can quantise the token itself (one launch less)
     fuse_quant = (self.fuse_quantize and isinstance(cache, Int8KVCacheGenerate)
                   and self._will_fuse(seqlen, cache.cache_k) and xk.dtype == torch.bfloat16
                   and xk.is_contiguous() and xv.is_contiguous())
     ret = cache.update(xk, xv, self.layer_id, defer_quantize=True) if fuse_quant \
-        else cache.update(xk, xv, self.layer_id)
+        else cache.update(xk, xv, self.layer_id, **rope_kw)
     if len(ret) == 4:  # int8 pages: (codes k, codes v, scale pages k, scale pages v)
       orig_keys, orig_values, k_scaler, v_scaler = ret
       new_key = new_value = new_k_scaler = new_v_scaler = None
@@ -118,7 +147,7 @@ class Int8KVAttentionKernel(AttentionKernel):
       new = dict(new_key=new_key, new_value=new_value, new_k_scaler=new_k_scaler,
                  new_v_scaler=new_v_scaler)
       if fuse_quant:
-        new.update(new_key_raw=xk, new_value_raw=xv, new_rounding=cache.rounding)
+        new.update(new_key_raw=xk, new_value_raw=xv, new_rounding=cache.rounding, new_key_rope=freqs_cis)
       return self._attend(xq, orig_keys, orig_values, k_scaler, v_scaler, mask, *args,
                           new_token=new)[0]
     existing_output, (existing_max, existing_denom) = self._attend(

@@ -19,12 +19,14 @@ def _rounding_code(rounding):
   raise ValueError(f"rounding must be 'trunc' or 'rne', got {rounding!r}")
 
 
-def quantize_kv(xk, xv, *, rounding="trunc", scale_heads=1, scale_dtype=None):
+def quantize_kv(xk, xv, *, rounding="trunc", scale_heads=1, scale_dtype=None, freqs_cis=None):
   """Quantises one token per slot: xk, xv (batch, heads, 1, dim).
 
   Returns (k_codes, v_codes, k_scale, v_scale); codes int8 of the input
   shape, scales (batch, scale_heads, 1, 1) in `scale_dtype` (default: the
-  input dtype).
+  input dtype).  With `freqs_cis` (the step's rotary factors, (batch, 1,
+  dim / 2) complex64) xk is taken unrotated and apply_rotary_emb
+  (jetstream_pt/layers.py:368-379) is applied to it in the same launch.
   """
   _ffi.dev(xk, "xk"), _ffi.dev(xv, "xv")
   b, h, t, d = xk.shape
@@ -40,5 +42,10 @@ def quantize_kv(xk, xv, *, rounding="trunc", scale_heads=1, scale_dtype=None):
       out_k_scale=_ffi.ptr(ks), out_v_scale=_ffi.ptr(vs), pos_count=b, batch=b, heads=h,
       seq=1, dim=d, in_dtype=_ffi.dtype_code(xk.dtype), scale_dtype=_ffi.dtype_code(sdt),
       scale_heads=scale_heads, rounding=_rounding_code(rounding))
+  rope = None
+  if freqs_cis is not None:
+    rope = _ffi.rope_factors(freqs_cis, b, d)
+    args.rope = _ffi.ptr(rope)
   _ffi.check(_ffi.lib.jpt_kv_append_quant_i8(args, _ffi.stream()))
+  del rope
   return kq, vq, ks, vs

@@ -23,5 +23,5 @@ installer pin jax 0.4.37) - in particular whether it applies 1/sqrt(head_dim).
 `oracle.attention.paged_attention` therefore takes `sm_scale` explicitly.
 """
 
-from . import attention, decode_state, insert, kv_cache, page_manager, quant  # noqa: F401
+from . import attention, decode_state, insert, kv_cache, page_manager, quant, rope  # noqa: F401
 from .env import Env  # noqa: F401
