@@ -148,6 +148,109 @@ __global__ void __launch_bounds__(256) prefill_insert_kernel(InsertParams p) {
   if (threadIdx.x < groups) store_from_f32(scale_out, scale_index(threadIdx.x), a.scale_dtype, s_scale[threadIdx.x]);
 }
 
+// The common quantising shape - bf16 prompt, heads * dim == 1024 - four tokens
+// a workgroup: a thread keeps its four elements of each token in registers
+// between the absmax pass and the quantise pass, so the prompt is read once
+// and four times as many bytes are in flight per workgroup.  Same op order.
+constexpr int kTokensPerBlock = 4;
+template <bool BF16_MATH>
+__global__ void __launch_bounds__(256) prefill_insert_quant4_kernel(InsertParams p) {
+  const jpt_prefill_insert_args& a = p.a;
+  const int t0 = blockIdx.x * kTokensPerBlock;
+  const bool is_v = blockIdx.y == 1;
+  const int layer = blockIdx.z;
+  const bool paged = a.page_ids != nullptr;
+  const int H = a.heads, D = a.dim;
+  const int rows = paged ? a.n_pages * a.page_size : a.tokens;
+  const int esz_scale = a.scale_dtype == JPT_F32 ? 4 : 2;
+  const uint16_t* src = static_cast<const uint16_t*>(is_v ? a.src_v : a.src_k) + layer * a.src_layer_stride;
+  char* dst = static_cast<char*>(is_v ? a.dst_v : a.dst_k) + layer * a.dst_layer_stride;
+  void* scale_out = static_cast<char*>(is_v ? a.v_scale : a.k_scale) + layer * a.scale_layer_stride * esz_scale;
+  const int i0 = 4 * threadIdx.x, h = i0 / D, d = i0 - h * D;
+  const int groups = a.scale_heads;
+  const int64_t head_stride = a.src_head_stride > 0 ? a.src_head_stride : static_cast<int64_t>(a.tokens) * D;
+
+  float x[kTokensPerBlock][4], m[kTokensPerBlock];
+  int64_t pool_row[kTokensPerBlock];  // dense: position in the slot's row; paged: row in the pool; -1: nothing to write
+#pragma unroll
+  for (int j = 0; j < kTokensPerBlock; ++j) {
+    const int t = t0 + j;
+    pool_row[j] = -1;
+    m[j] = 0.f;
+    x[j][0] = x[j][1] = x[j][2] = x[j][3] = 0.f;
+    if (t >= rows) continue;
+    if (paged) {
+      const int page = a.page_ids[t / a.page_size];
+      if (page >= 0 && page < a.total_pages) pool_row[j] = static_cast<int64_t>(page) * a.page_size + t % a.page_size;
+    } else {
+      const int at = (a.start + t) % a.seq;
+      pool_row[j] = at < 0 ? at + a.seq : at;
+    }
+    if (t < a.tokens) {
+      const uint2 raw = *reinterpret_cast<const uint2*>(src + h * head_stride + static_cast<int64_t>(t) * D + d);
+      x[j][0] = __uint_as_float(raw.x << 16);
+      x[j][1] = __uint_as_float(raw.x & 0xffff0000u);
+      x[j][2] = __uint_as_float(raw.y << 16);
+      x[j][3] = __uint_as_float(raw.y & 0xffff0000u);
+      m[j] = fmaxf(fmaxf(fabsf(x[j][0]), fabsf(x[j][1])), fmaxf(fabsf(x[j][2]), fabsf(x[j][3])));
+    }
+  }
+  __shared__ float s_red[kTokensPerBlock][4];
+  if (groups == 1) {
+#pragma unroll
+    for (int j = 0; j < kTokensPerBlock; ++j) {
+      for (int off = 32; off > 0; off >>= 1) m[j] = fmaxf(m[j], __shfl_xor(m[j], off));
+      if ((threadIdx.x & 63) == 0) s_red[j][threadIdx.x >> 6] = m[j];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kTokensPerBlock; ++j)
+      m[j] = fmaxf(fmaxf(s_red[j][0], s_red[j][1]), fmaxf(s_red[j][2], s_red[j][3]));
+  } else {
+    // a head's D / 4 threads are consecutive; D / 4 is a power of two <= 64
+#pragma unroll
+    for (int j = 0; j < kTokensPerBlock; ++j)
+      for (int off = D / 8; off > 0; off >>= 1) m[j] = fmaxf(m[j], __shfl_xor(m[j], off));
+  }
+#pragma unroll
+  for (int j = 0; j < kTokensPerBlock; ++j) {
+    if (pool_row[j] < 0) continue;
+    const int64_t row = paged ? static_cast<int64_t>(h) * a.total_pages * a.page_size + pool_row[j]
+                              : (static_cast<int64_t>(a.slot) * H + h) * a.seq + pool_row[j];
+    uint32_t* out = reinterpret_cast<uint32_t*>(dst + row * D + d);
+    if (t0 + j >= a.tokens) {  // paged only: the tail of the last page is zero-filled
+      *out = 0u;
+      continue;
+    }
+    float amax = m[j];
+    if (a.rounding == JPT_ROUND_RNE) amax = fmaxf(amax, rnd<BF16_MATH>(1e-5f));
+    const float s = rnd<BF16_MATH>(amax / 127.0f);
+    int code[4];
+    if (a.rounding == JPT_ROUND_TRUNC) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float q = rnd<BF16_MATH>(x[j][i] / s);
+        code[i] = (q != q) ? 0 : static_cast<int>(q);
+      }
+    } else {
+      const float r = rnd<BF16_MATH>(1.0f / s);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float q = rnd<BF16_MATH>(x[j][i] * r);
+        code[i] = static_cast<int>(fminf(fmaxf(rintf(q), -128.f), 127.f));
+      }
+    }
+    *out = (static_cast<uint32_t>(code[0]) & 0xffu) | ((static_cast<uint32_t>(code[1]) & 0xffu) << 8) |
+           ((static_cast<uint32_t>(code[2]) & 0xffu) << 16) | (static_cast<uint32_t>(code[3]) << 24);
+    if (groups == 1 ? threadIdx.x == 0 : d == 0) {
+      const int g = groups == 1 ? 0 : h;
+      const int64_t idx = paged ? static_cast<int64_t>(g) * a.total_pages * a.page_size + pool_row[j]
+                                : (static_cast<int64_t>(a.slot) * groups + g) * a.seq + pool_row[j];
+      store_from_f32(scale_out, idx, a.scale_dtype, s);
+    }
+  }
+}
+
 }  // namespace
 }  // namespace jpt
 
@@ -189,6 +292,18 @@ extern "C" int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void*
   InsertParams p{*args};
   if (p.a.n_layers <= 0) p.a.n_layers = 1;
   JPT_REQUIRE(p.a.n_layers <= 65535, "n_layers out of range");
+  const int d4 = a.dim / 4;
+  const bool four = quant && a.in_dtype == JPT_BF16 && a.heads * a.dim == 1024 &&
+                    (a.scale_heads == 1 || (d4 <= 64 && (d4 & (d4 - 1)) == 0)) && aligned(a.src_k, 8) &&
+                    aligned(a.src_v, 8) && (a.src_head_stride == 0 || a.src_head_stride % 4 == 0);
+  if (four) {
+    dim3 grid4((rows + kTokensPerBlock - 1) / kTokensPerBlock, 2, p.a.n_layers);
+    if (a.scale_dtype == JPT_BF16)
+      hipLaunchKernelGGL(prefill_insert_quant4_kernel<true>, grid4, dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    else
+      hipLaunchKernelGGL(prefill_insert_quant4_kernel<false>, grid4, dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    return launch_status("prefill_insert_quant4_kernel");
+  }
   dim3 grid(rows, 2, p.a.n_layers);
   if (quant && a.scale_dtype == JPT_BF16)
     hipLaunchKernelGGL(prefill_insert_kernel<true>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), p);

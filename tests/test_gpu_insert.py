@@ -91,6 +91,12 @@ def test_llama3_shaped_quantised_insert_fp32_scales():
   run_both(False, True, (4, 8, 2048, 128, 2), prompt=1024, seq_len=1000, slot=3, scale_dtype=torch.float32)
 
 
+@pytest.mark.parametrize("ring,current_position,seq_len,prompt", [(False, 0, 37, 40), (True, 250, 61, 64), (True, 3, 5, 8)])
+def test_llama3_shaped_quantised_insert_bf16_scales_ragged_counts(ring, current_position, seq_len, prompt):
+  # token counts that are not multiples of the four tokens a workgroup takes, ring wrap included
+  run_both(ring, True, (3, 8, 256, 128, 2), prompt=prompt, seq_len=seq_len, slot=1, current_position=current_position)
+
+
 def test_float32_prefix_into_float32_quantiser():
   run_both(False, True, (2, 4, 64, 16, 1), prompt=32, seq_len=30, slot=0, scale_dtype=torch.float32,
            prefix_dtype=torch.float32)
