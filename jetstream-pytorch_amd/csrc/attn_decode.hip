@@ -284,7 +284,9 @@ int32_t attn_fast_launch(const jpt_attn_args& a, AttnMode mode, hipStream_t stre
   else decode::launch_decode_bf16(p, mode == kPaged, blocks, stream);
   int32_t st = launch_status("attn_decode_kernel");
   if (st != JPT_OK) return st;
-  hipLaunchKernelGGL(attn_merge_kernel, dim3(a.batch * a.kv_heads), dim3(256), 0, stream, p);
+  // 16 lanes a row: only as many waves as the rows need
+  const unsigned merge_threads = static_cast<unsigned>((rows * 16 + 63) / 64 * 64);
+  hipLaunchKernelGGL(attn_merge_kernel, dim3(a.batch * a.kv_heads), dim3(merge_threads), 0, stream, p);
   return launch_status("attn_merge_kernel");
 }
 

@@ -150,6 +150,29 @@ __device__ __forceinline__ T load_uniform(const T* p) {
   return *(constant_ptr)p;
 }
 
+// Maximum over the wave's 64 lanes, the same value in every lane.  Data-parallel
+// primitives inside the 16-lane rows (quad swaps, then the row's halves and the
+// row mirrored), four lane reads across the rows: no LDS round trips.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float row_max(float v) {
+  v = fmaxf(v, dpp_move<0xB1>(v));   // quad_perm [1, 0, 3, 2]
+  v = fmaxf(v, dpp_move<0x4E>(v));   // quad_perm [2, 3, 0, 1]
+  v = fmaxf(v, dpp_move<0x141>(v));  // row_half_mirror
+  v = fmaxf(v, dpp_move<0x140>(v));  // row_mirror
+  return v;
+}
+__device__ __forceinline__ float rows_max(float r) {
+  const int bits = __builtin_bit_cast(int, r);
+  const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0));
+  const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16));
+  const float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32));
+  const float d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48));
+  return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding)
 constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
 
@@ -734,7 +757,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   // accumulates it; `valid` positions of the tile count (all of them when
   // `full_tag` says so).
   int cur_slot = 0, cur_h = 0;  // of the item being consumed
-  // Quantises the new token of slot cur_slot, whose kv_heads bf16 rows lie one
+  // Quantising the new token of slot cur_slot, whose kv_heads bf16 rows lie one
   // after another in `area` (the tile's key or value area): arithmetic and
   // rounding of jpt_kv_append_quant_i8, each step rounded to the scale dtype.
   // The absmax runs over every head (one scale per token) or over head cur_h;
@@ -743,9 +766,11 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   // item, with per-head scales) stores the scale.
   // `rope`: NULL, or the slot's (cos, sin) factors: the rows are rotated pair by
   // pair first (keys only), rounded to bf16 as the separate rotary op would.
-  auto quantise_new = [&](char* area, int8_t* stash, void* scale_out, const float* rope) -> float {
-    constexpr bool kBf16Math = SCALE == kScaleBF16;
-    auto rnd = [](float x) { return kBf16Math ? round_to_bf16(x) : x; };
+  // Two steps, so that the key's and the value's reductions overlap: new_absmax
+  // leaves the lane's two elements of head cur_h in x0, x1 and returns the
+  // lane's share of the absmax; new_encode takes the wave-wide absmax.
+  constexpr bool kBf16Math = SCALE == kScaleBF16;
+  auto new_absmax = [&](const char* area, const float* rope, float& x0, float& x1) -> float {
     auto rotate = [](float& x, float& y, float c, float s) {
 #pragma clang fp contract(off)  // the products are rounded before they are combined
       const float xc = x * c, ys = y * s, xs = x * s, yc = y * c;
@@ -755,7 +780,8 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       y = round_to_bf16(im);
     };
     const uint32_t pair = *reinterpret_cast<const uint32_t*>(area + cur_h * (kD * 2) + lane * 4);
-    float x0 = __uint_as_float(pair << 16), x1 = __uint_as_float(pair & 0xffff0000u);
+    x0 = __uint_as_float(pair << 16);
+    x1 = __uint_as_float(pair & 0xffff0000u);
     if (rope) {  // the lane's elements 2 * lane, 2 * lane + 1 of the head are pair number `lane`
       const float2 cs = *reinterpret_cast<const float2*>(rope + 2 * lane);
       rotate(x0, x1, cs.x, cs.y);
@@ -785,8 +811,10 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         for (int i = 0; i < 16; ++i) m = fmaxf(m, fabsf(f[i]));
       }
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    return m;
+  };
+  auto new_encode = [&](char* area, int8_t* stash, void* scale_out, float x0, float x1, float m) -> float {
+    auto rnd = [](float x) { return kBf16Math ? round_to_bf16(x) : x; };
     if (a.new_rounding == JPT_ROUND_RNE) m = fmaxf(m, rnd(1e-5f));
     const float sc = rnd(m / 127.0f);
     int c0, c1;
@@ -801,7 +829,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     }
     const uint16_t codes = static_cast<uint16_t>((c0 & 0xff) | ((c1 & 0xff) << 8));
     // row 0 of the tile: piece p sits at piece slot p ^ 0.  Every lane has read
-    // its raw elements above, before any lane's codes land on them.
+    // its raw elements before any lane's codes land on them.
     *reinterpret_cast<uint16_t*>(area + lane * 2) = codes;
     *reinterpret_cast<uint16_t*>(stash + (static_cast<int64_t>(cur_slot) * a.kv_heads + cur_h) * kD + lane * 2) = codes;
     if (lane == 0 && (a.scale_heads != 1 || cur_h == 0)) {
@@ -827,8 +855,13 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     const bool quant_here = !FULL && is_new && quant_new;
     if (quant_here) {
       const float* rope = a.new_k_rope ? a.new_k_rope + static_cast<int64_t>(cur_slot) * kD : nullptr;
-      new_ks = quantise_new(slot, static_cast<int8_t*>(const_cast<void*>(a.new_k)), const_cast<void*>(a.new_k_scale), rope);
-      new_vs = quantise_new(slot + C::kTileBytes, static_cast<int8_t*>(const_cast<void*>(a.new_v)), const_cast<void*>(a.new_v_scale), nullptr);
+      float k0, k1, v0, v1;
+      const float mk = new_absmax(slot, rope, k0, k1), mv = new_absmax(slot + C::kTileBytes, nullptr, v0, v1);
+      const float rk = row_max(mk), rv = row_max(mv);  // both reductions in flight together
+      new_ks = new_encode(slot, static_cast<int8_t*>(const_cast<void*>(a.new_k)), const_cast<void*>(a.new_k_scale), k0, k1,
+                          rows_max(rk));
+      new_vs = new_encode(slot + C::kTileBytes, static_cast<int8_t*>(const_cast<void*>(a.new_v)),
+                          const_cast<void*>(a.new_v_scale), v0, v1, rows_max(rv));
     }
     T tile;
     tile.read(slot, slot + C::kTileBytes, r, g, pos);
