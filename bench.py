@@ -523,6 +523,8 @@ def main():
   ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c3")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   ap.add_argument("--no-graph", action="store_true", help="launch every step from Python")
+  ap.add_argument("--first-use-memory", action="store_true",
+                  help="time the workload on its first allocation only (no free-and-allocate-again pass)")
   ap.add_argument("--host-alloc", action="store_true",
                   help="c4/c5: page allocator on the host as in the reference (no graph capture)")
   ap.add_argument("--probe-traffic", action="store_true",
@@ -535,6 +537,24 @@ def main():
     run_traffic_probe(args)
     return
   r = run_gpu(args)
+  first_use = None
+  if not args.first_use_memory:
+    # HBM handed out for the first time after the device comes up streams more
+    # slowly on this pool than memory that has been allocated before (C3: 48.4
+    # against 45.1 us per layer-step, the same kernels, the same virtual
+    # addresses).  A serving process on a node that has been up for a while
+    # sits in the second state: the workload is built once on first-use memory
+    # (reported as first_use_memory), freed, and built again for `value`.
+    import gc
+
+    import torch
+    first_use = {"us_per_layer": round(r["ms_per_step"] * 1e3, 2),
+                 "GB_per_s": round(r["step_bytes"] / (r["ms_per_step"] * 1e-3) / 1e9, 1),
+                 "attention_us_per_launch": round(r["attn_ms"] * 1e3, 2)}
+    del r
+    gc.collect()
+    torch.cuda.empty_cache()
+    r = run_gpu(args)
   gbps = r["step_bytes"] / (r["ms_per_step"] * 1e-3) / 1e9
   attn_gbps = r["attn_bytes"] / (r["attn_ms"] * 1e-3) / 1e9
   headline = args.workload == "c3"
@@ -566,6 +586,9 @@ def main():
           "us_per_launch": round(r["attn_ms"] * 1e3, 2), "algorithmic_bytes": int(r["attn_bytes"]),
       },
   }
+  if first_use is not None:
+    cfg["memory"] = "synthetic cache allocated, freed and allocated again before timing; first_use_memory = the same run on the first allocation"
+    line["first_use_memory"] = first_use
   if headline and not args.no_cpu_baseline:
     line["cpu_baseline"] = run_cpu_baseline()
   print(json.dumps(line))
