@@ -456,16 +456,18 @@ def run_traffic_probe(args):
   vs = torch.empty_like(ks).uniform_(0.005, 0.05)
   g = torch.Generator(device=DEV).manual_seed(SEED)
   xq = torch.randn((B, HQ, 1, D), generator=g, device=DEV).to(torch.bfloat16)
-  nk = torch.empty((B, HKV, 1, D), dtype=torch.int8, device=DEV).random_(-127, 128)
-  nv = torch.empty_like(nk).random_(-127, 128)
-  nks = torch.empty((B, 1, 1, 1), device=DEV).uniform_(0.005, 0.05)
-  nvs = torch.empty_like(nks).uniform_(0.005, 0.05)
+  xk = torch.randn((B, HKV, 1, D), generator=g, device=DEV).to(torch.bfloat16)
+  xv = torch.randn((B, HKV, 1, D), generator=g, device=DEV).to(torch.bfloat16)
+  nk = torch.empty((B, HKV, 1, D), dtype=torch.int8, device=DEV)  # written by the launch
+  nv = torch.empty_like(nk)
+  nks = torch.empty((B, 1, 1, 1), device=DEV)
+  nvs = torch.empty_like(nks)
   plan, _ = ak.precompute_ragged_block_indices(lengths, B, HQ, HKV, S)
   src = torch.empty(PROBE_COPY_BYTES // 4, dtype=torch.float32, device=DEV).normal_()
   dst = torch.empty_like(src)
   for i in range(8):
     ak.ragged_mha(xq, k, v, i % nl, None, plan.lengths, plan, None, ks, vs, new_key=nk, new_value=nv,
-                  new_k_scaler=nks, new_v_scaler=nvs)
+                  new_k_scaler=nks, new_v_scaler=nvs, new_key_raw=xk, new_value_raw=xv)
     dst.copy_(src)
   torch.cuda.synchronize()
   print(json.dumps({"probe": "traffic", "attention_launches": 8, "copies": 8,
