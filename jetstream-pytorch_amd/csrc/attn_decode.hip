@@ -43,9 +43,14 @@ int32_t env_int(const char* name, int32_t fallback) {
   return t > 0 ? t : fallback;
 }
 
-// Work items (chunk x KV head) the planner aims for.
+int32_t persistent_blocks();
+
+// Work items (chunk x KV head) the planner aims for: five for every four
+// workers.  An item costs a few microseconds beyond its tiles (query rows,
+// fold, output or partial), so chunks are made about as long as a worker's
+// share of the positions, and the sort-and-deal of the plan evens out the rest.
 int32_t target_items() {
-  static int32_t v = env_int("JPT_ATTN_TARGET_ITEMS", 2048);
+  static int32_t v = env_int("JPT_ATTN_TARGET_ITEMS", persistent_blocks() * 5 / 4);
   return v;
 }
 
