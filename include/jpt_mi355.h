@@ -431,6 +431,20 @@ int32_t jpt_decode_advance(void* mask, int32_t mask_dtype, int64_t mask_stride,
                            int32_t current_position, int32_t update_mask,
                            int32_t advance, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Engine.precompute_ragged_block_indices (engine.py:674-729): for every grid
+ * cell (slot b, block i) of the reference's ring-aware ragged kernel, the
+ * (slot, block) it works on.  start, input_pos (batch) int32 on the device,
+ * end = (start + input_pos) % cache_len; b_next, i_next (batch, cache_len /
+ * block_size) int32.  The attention entry points above do not read these
+ * tables (nor does the reference's live kernel, attention_kernel.py:561-579);
+ * provided for callers that carry them in their decode state.
+ * ---------------------------------------------------------------------- */
+int32_t jpt_ragged_block_indices(const int32_t* start, const int32_t* input_pos,
+                                 int32_t batch, int32_t cache_len,
+                                 int32_t block_size, int32_t* b_next,
+                                 int32_t* i_next, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

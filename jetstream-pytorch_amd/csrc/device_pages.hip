@@ -203,6 +203,36 @@ decode_advance_kernel(T* mask, int64_t mask_stride, int32_t* input_pos, int32_t*
   }
 }
 
+// One thread per cell (slot b, block i) of the reference's block-index tables:
+// the block the ring-aware ragged kernel of the reference would work on from
+// that grid cell (engine.py:674-729).  end = (start + input_pos) % cache_len.
+__global__ void __launch_bounds__(kThreads)
+ragged_block_indices_kernel(const int32_t* start, const int32_t* input_pos, int batch, int cache_len, int bk,
+                            int num_bk, int32_t* b_next, int32_t* i_next) {
+  const int cell = blockIdx.x * blockDim.x + threadIdx.x;
+  if (cell >= batch * num_bk) return;
+  const int b = cell / num_bk, i = cell - b * num_bk;
+  const int s = start[b];
+  const int e = static_cast<int>((static_cast<int64_t>(s) + input_pos[b]) % cache_len);
+  const bool last = b == batch - 1;
+  // where a finished slot hands over: block 0 of the next slot; the last slot
+  // stays on its own last block that can hold a live position
+  const int hand_b = last ? b : b + 1;
+  const int hand_i = last ? (s < e ? (e - 1) / bk : (cache_len - 1) / bk) : 0;
+  int nb = b, ni = i;
+  if (s < e) {
+    if (i * bk >= e) { nb = hand_b; ni = hand_i; }
+    if ((i + 1) * bk <= s) ni = s / bk;
+  } else if (s == e) {
+    nb = hand_b;
+    ni = hand_i;
+  } else if (i * bk >= e && (i + 1) * bk <= s) {
+    ni = s / bk;
+  }
+  b_next[cell] = nb;
+  i_next[cell] = ni;
+}
+
 int32_t check_dpam(const jpt_dpam* pam) {
   JPT_REQUIRE(pam != nullptr, "pam is NULL");
   JPT_REQUIRE(pam->state && pam->ring && pam->page_indices && pam->lengths && pam->n_alloc && pam->update_indices,
@@ -284,6 +314,20 @@ int32_t jpt_decode_advance(void* mask, int32_t mask_dtype, int64_t mask_stride, 
     hipLaunchKernelGGL(decode_advance_kernel<float>, grid, dim3(kThreads), 0, s, static_cast<float*>(mask),
                        mask_stride, input_pos, lens, batch, seq, ring_buffer, current_position, update_mask, advance);
   return launch_status("decode_advance_kernel");
+}
+
+int32_t jpt_ragged_block_indices(const int32_t* start, const int32_t* input_pos, int32_t batch, int32_t cache_len,
+                                 int32_t block_size, int32_t* b_next, int32_t* i_next, void* stream) {
+  using namespace jpt;
+  JPT_REQUIRE(start && input_pos && b_next && i_next, "NULL argument");
+  JPT_REQUIRE(batch > 0 && cache_len > 0 && block_size > 0, "batch, cache_len and block_size must be positive");
+  JPT_REQUIRE(cache_len % block_size == 0, "cache_len must be a multiple of block_size");
+  const int num_bk = cache_len / block_size;
+  JPT_REQUIRE(static_cast<int64_t>(batch) * num_bk <= INT32_MAX, "table too large");
+  const dim3 grid((batch * num_bk + kThreads - 1) / kThreads);
+  hipLaunchKernelGGL(ragged_block_indices_kernel, grid, dim3(kThreads), 0, static_cast<hipStream_t>(stream), start,
+                     input_pos, batch, cache_len, block_size, num_bk, b_next, i_next);
+  return launch_status("ragged_block_indices_kernel");
 }
 
 }  // extern "C"

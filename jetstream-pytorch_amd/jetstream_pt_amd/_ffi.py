@@ -139,6 +139,7 @@ _sig("jpt_dpam_reserve_insert", _i32, _c.POINTER(Dpam), _vp, _vp, _i32, _i32, _i
 _sig("jpt_dpam_free", _i32, _c.POINTER(Dpam), _vp, _i32, _i32, _vp)
 _sig("jpt_dpam_decode_step", _i32, _c.POINTER(Dpam), _vp, _vp)
 _sig("jpt_decode_advance", _i32, _vp, _i32, _i64, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp)
+_sig("jpt_ragged_block_indices", _i32, _vp, _vp, _i32, _i32, _i32, _vp, _vp, _vp)
 
 EXPORTS = (
     "jpt_version", "jpt_last_error", "jpt_kv_scatter_lines",
@@ -150,6 +151,7 @@ EXPORTS = (
     "jpt_pam_fill_new_pages", "jpt_pam_page_token_indices", "jpt_pam_free",
     "jpt_pam_free_count", "jpt_paged_append_dev", "jpt_dpam_init", "jpt_dpam_reserve_insert",
     "jpt_dpam_free", "jpt_dpam_decode_step", "jpt_decode_advance", "jpt_rope",
+    "jpt_ragged_block_indices",
 )
 
 

@@ -51,3 +51,24 @@ def finish_step(mask, input_pos, lens=None, *, ring_buffer=False, current_positi
   order of generate_impl, one launch."""
   _advance(mask, input_pos, lens, ring_buffer, current_position, True, True)
   return mask, input_pos, lens
+
+
+def ragged_block_indices(start, input_pos, cache_len, block_size):
+  """The reference's Engine.precompute_ragged_block_indices (engine.py:674-729)
+  on device tensors: start, input_pos (batch) int32; returns (b_next, i_next),
+  each (batch, cache_len // block_size) int32.  The attention entry points of
+  this package do not read them (the reference's live kernel does not either);
+  for callers whose decode state carries the tables."""
+  start = _ffi.dev(start, "start")
+  input_pos = _ffi.dev(input_pos, "input_pos")
+  if start.dtype != torch.int32 or input_pos.dtype != torch.int32 or start.numel() != input_pos.numel():
+    raise ValueError("start and input_pos must be int32 device tensors of one entry per slot")
+  if cache_len % block_size != 0:
+    raise ValueError("cache_len must be a multiple of block_size")
+  batch = start.numel()
+  b_next = torch.empty((batch, cache_len // block_size), dtype=torch.int32, device=start.device)
+  i_next = torch.empty_like(b_next)
+  _ffi.check(_ffi.lib.jpt_ragged_block_indices(
+      _ffi.ptr(start.contiguous()), _ffi.ptr(input_pos.contiguous()), batch, int(cache_len), int(block_size),
+      _ffi.ptr(b_next), _ffi.ptr(i_next), _ffi.stream()))
+  return b_next, i_next

@@ -27,3 +27,35 @@ def advance(input_pos, lens, cache_len, ring_buffer=False):
     return input_pos + 1, lens + 1
   return (np.where(input_pos == 0, 0, input_pos + 1 % cache_len),
           np.where(lens == 0, 0, lens + 1 % cache_len))
+
+
+def ragged_block_indices(start, input_pos, cache_len, block_size):
+  """engine.py:674-729: the (batch, cache_len // block_size) tables
+  (b_next, i_next) that tell the reference's ring-aware ragged kernel, for grid
+  cell (slot b, block i), which (slot, block) to work on.  The live ragged
+  kernel of the reference ignores them (attention_kernel.py:561-579 calls the
+  left-aligned one); restated for completeness, same where-expressions."""
+  start = np.asarray(start).astype(np.int64)
+  end = (start + np.asarray(input_pos).astype(np.int64)) % cache_len
+  batch = start.shape[0]
+  bk = block_size
+  num_bk = cache_len // bk
+  b = np.arange(batch).reshape(batch, 1)
+  i = np.broadcast_to(np.arange(num_bk).reshape(1, num_bk), (batch, num_bk))
+  start = start.reshape(batch, 1)
+  end = end.reshape(batch, 1)
+  last_slot = b == batch - 1
+  last_good_block = np.where(start < end, (end - 1) // bk, (cache_len - 1) // bk)
+  next_b = np.where(last_slot, b, b + 1)
+  next_i = np.where(last_slot, last_good_block, 0)
+  # start < end: stay while the block overlaps [start, end)
+  past = i * bk >= end
+  t_b = np.where(past, next_b, b)
+  t_i = np.where(past, next_i, i)
+  t_i = np.where((i + 1) * bk <= start, start // bk, t_i)
+  # start > end: stay unless the block lies inside the gap [end, start)
+  f_b = np.broadcast_to(b, (batch, num_bk))
+  f_i = np.where((i * bk >= end) & ((i + 1) * bk <= start), start // bk, i)
+  b_next = np.where(start < end, t_b, np.where(start == end, next_b, f_b))
+  i_next = np.where(start < end, t_i, np.where(start == end, next_i, f_i))
+  return b_next.astype(np.int32), i_next.astype(np.int32)

@@ -136,6 +136,31 @@ def test_decode_state_bookkeeping(ring, dtype):
   assert np.array_equal(gp2.cpu().numpy(), want_pos)
 
 
+@pytest.mark.parametrize("batch,cache_len,bk", [(6, 64, 16), (9, 96, 8), (128, 8192, 512), (1, 32, 32)])
+def test_ragged_block_index_tables(batch, cache_len, bk):
+  """engine.py:674-729 on the device: integer tables, exact."""
+  from jetstream_pt_amd import decode_state
+  rng = np.random.default_rng(batch + bk)
+  for _ in range(5):
+    start = rng.integers(0, cache_len, batch).astype(np.int32)
+    pos = rng.integers(0, cache_len, batch).astype(np.int32)
+    start[0] = (start[0] // bk) * bk
+    pos[batch // 2] = 0  # an empty slot
+    pos[-1] = (cache_len - start[-1]) % cache_len  # the last slot's run ends at the cache end
+    want_b, want_i = ods.ragged_block_indices(start, pos, cache_len, bk)
+    got_b, got_i = decode_state.ragged_block_indices(
+        torch.from_numpy(start).to(DEV), torch.from_numpy(pos).to(DEV), cache_len, bk)
+    assert got_b.shape == (batch, cache_len // bk)
+    assert np.array_equal(got_b.cpu().numpy(), want_b) and np.array_equal(got_i.cpu().numpy(), want_i)
+  # left-aligned slots (no ring buffer): start = 0
+  zero = torch.zeros(batch, dtype=torch.int32, device=DEV)
+  want_b, want_i = ods.ragged_block_indices(np.zeros(batch, np.int32), pos, cache_len, bk)
+  got_b, got_i = decode_state.ragged_block_indices(zero, torch.from_numpy(pos).to(DEV), cache_len, bk)
+  assert np.array_equal(got_b.cpu().numpy(), want_b) and np.array_equal(got_i.cpu().numpy(), want_i)
+  with pytest.raises(ValueError):
+    decode_state.ragged_block_indices(zero, zero, cache_len, bk + 1)
+
+
 def _paged_setup(int8, seed):
   """Two identical paged caches, one driven by the host allocator, one by the
   device allocator, with the same prompts inserted."""
