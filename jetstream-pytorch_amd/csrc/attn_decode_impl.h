@@ -53,7 +53,10 @@ typedef const __attribute__((address_space(1))) void* global_ptr;
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
 #ifndef JPT_ATTN_EXPERIMENT_CUT
-#define JPT_ATTN_EXPERIMENT_CUT 0  // development: stop a tile's work early (timing experiments only)
+// Development builds for timing experiments only (results are wrong): 1, 2 stop a
+// tile's work early; 3 skips an item's fold and output; 4 only the fold by the
+// last consumer to arrive; 5 the conversion of the query operand.
+#define JPT_ATTN_EXPERIMENT_CUT 0
 #endif
 #ifndef JPT_ATTN_CONSUMERS
 #define JPT_ATTN_CONSUMERS 3
@@ -975,6 +978,9 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   // consumer to arrive folds the parts and writes the slot's output (one
   // chunk) or parks the chunk's partial (several).
   auto finish_item = [&](const Item& it, int seq) -> bool {
+#if JPT_ATTN_EXPERIMENT_CUT == 3
+    return true;
+#endif
     const int buf = seq % C::kFoldBufs;
     // the buffer's previous item must have been folded out of it
     if (!wait_for(&sm_folded[buf], seq / C::kFoldBufs)) return false;
@@ -996,6 +1002,13 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       arrived = __hip_atomic_fetch_add(&sm_arrived[buf], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_WORKGROUP);
     arrived = __builtin_amdgcn_readfirstlane(arrived);
     if (arrived != kConsumers - 1) return true;
+#if JPT_ATTN_EXPERIMENT_CUT == 4
+    if (lane == 0) {
+      __hip_atomic_store(&sm_arrived[buf], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_fetch_add(&sm_folded[buf], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    return true;
+#endif
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     const int64_t q_row0 = (static_cast<int64_t>(it.slot) * a.q_heads + it.h * p.rep) * a.q_rows;
     float* part = p.partials + (static_cast<int64_t>(it.part) * a.kv_heads + it.h) * R * kPartFloats;
@@ -1069,7 +1082,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         u[kk] = make_uint4(0, 0, 0, 0);
         if (r < R) u[kk] = *reinterpret_cast<const uint4*>(&sm_q[qb][r][32 * g + 8 * kk]);
       }
-      if (T::kBias == 0.f) {
+      if (T::kBias == 0.f || JPT_ATTN_EXPERIMENT_CUT == 5) {
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) qop[kk] = __builtin_bit_cast(Op, u[kk]);
       } else {
