@@ -170,30 +170,40 @@ __global__ void __launch_bounds__(256) prefill_insert_quant4_kernel(InsertParams
   const int groups = a.scale_heads;
   const int64_t head_stride = a.src_head_stride > 0 ? a.src_head_stride : static_cast<int64_t>(a.tokens) * D;
 
+  // All four tokens' loads are issued before anything waits for one of them
+  // (addresses clamped into the prompt, results masked afterwards), and the
+  // page ids likewise: one memory round trip a workgroup, not one a token.
+  uint2 raw[kTokensPerBlock];
+#pragma unroll
+  for (int j = 0; j < kTokensPerBlock; ++j) {
+    const int t = min(t0 + j, a.tokens - 1);
+    raw[j] = *reinterpret_cast<const uint2*>(src + h * head_stride + static_cast<int64_t>(t) * D + d);
+  }
+  int page_of[kTokensPerBlock];
+#pragma unroll
+  for (int j = 0; j < kTokensPerBlock; ++j)
+    page_of[j] = paged ? a.page_ids[min(t0 + j, rows - 1) / a.page_size] : 0;
   float x[kTokensPerBlock][4], m[kTokensPerBlock];
   int64_t pool_row[kTokensPerBlock];  // dense: position in the slot's row; paged: row in the pool; -1: nothing to write
 #pragma unroll
   for (int j = 0; j < kTokensPerBlock; ++j) {
     const int t = t0 + j;
     pool_row[j] = -1;
-    m[j] = 0.f;
-    x[j][0] = x[j][1] = x[j][2] = x[j][3] = 0.f;
-    if (t >= rows) continue;
-    if (paged) {
-      const int page = a.page_ids[t / a.page_size];
-      if (page >= 0 && page < a.total_pages) pool_row[j] = static_cast<int64_t>(page) * a.page_size + t % a.page_size;
-    } else {
-      const int at = (a.start + t) % a.seq;
-      pool_row[j] = at < 0 ? at + a.seq : at;
+    if (t < rows) {
+      if (paged) {
+        const int page = page_of[j];
+        if (page >= 0 && page < a.total_pages) pool_row[j] = static_cast<int64_t>(page) * a.page_size + t % a.page_size;
+      } else {
+        const int at = (a.start + t) % a.seq;
+        pool_row[j] = at < 0 ? at + a.seq : at;
+      }
     }
-    if (t < a.tokens) {
-      const uint2 raw = *reinterpret_cast<const uint2*>(src + h * head_stride + static_cast<int64_t>(t) * D + d);
-      x[j][0] = __uint_as_float(raw.x << 16);
-      x[j][1] = __uint_as_float(raw.x & 0xffff0000u);
-      x[j][2] = __uint_as_float(raw.y << 16);
-      x[j][3] = __uint_as_float(raw.y & 0xffff0000u);
-      m[j] = fmaxf(fmaxf(fabsf(x[j][0]), fabsf(x[j][1])), fmaxf(fabsf(x[j][2]), fabsf(x[j][3])));
-    }
+    const bool live = t < a.tokens;
+    x[j][0] = live ? __uint_as_float(raw[j].x << 16) : 0.f;
+    x[j][1] = live ? __uint_as_float(raw[j].x & 0xffff0000u) : 0.f;
+    x[j][2] = live ? __uint_as_float(raw[j].y << 16) : 0.f;
+    x[j][3] = live ? __uint_as_float(raw[j].y & 0xffff0000u) : 0.f;
+    m[j] = fmaxf(fmaxf(fabsf(x[j][0]), fabsf(x[j][1])), fmaxf(fabsf(x[j][2]), fabsf(x[j][3])));
   }
   __shared__ float s_red[kTokensPerBlock][4];
   if (groups == 1) {
@@ -293,7 +303,7 @@ extern "C" int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void*
   if (p.a.n_layers <= 0) p.a.n_layers = 1;
   JPT_REQUIRE(p.a.n_layers <= 65535, "n_layers out of range");
   const int d4 = a.dim / 4;
-  const bool four = quant && a.in_dtype == JPT_BF16 && a.heads * a.dim == 1024 &&
+  const bool four = quant && a.tokens > 0 && a.in_dtype == JPT_BF16 && a.heads * a.dim == 1024 &&
                     (a.scale_heads == 1 || (d4 <= 64 && (d4 & (d4 - 1)) == 0)) && aligned(a.src_k, 8) &&
                     aligned(a.src_v, 8) && (a.src_head_stride == 0 || a.src_head_stride % 4 == 0);
   if (four) {
