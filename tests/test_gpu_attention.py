@@ -97,6 +97,29 @@ def test_ragged_fast_kernel_vs_closed_form(kind, hq, hkv, lens_name):
   check_out(o.reshape(b, hq, 1, d), OA.reshape_outputs(rep, ro)[0], "vs reference recurrence")
 
 
+@pytest.mark.parametrize("kind", ["int8", "bf16"])
+def test_ragged_very_large_batch(kind):
+  """1100 slots x 32 KV heads: more work items per worker than the kernel keeps
+  listed in LDS, so the later ones are fetched as they are reached."""
+  from jetstream_pt_amd import attention_kernel as ak
+  g = torch.Generator().manual_seed(312)
+  rng = np.random.default_rng(312)
+  b, hq, hkv, s, d = 1100, 32, 32, 128, 128
+  lens = rng.integers(0, s + 1, b).astype(np.int32)
+  lens[:8] = [0, 1, 31, 32, 33, s, s - 1, 2]
+  end = torch.from_numpy(lens)
+  q = rnd(g, (b, hq, 1, d))
+  if kind == "int8":
+    k, v, ks, vs = int8_cache(g, b, hkv, s, d)
+  else:
+    k, v, ks, vs = rnd(g, (b, hkv, s, d)), rnd(g, (b, hkv, s, d)), None, None
+  wo, wm, wl = OA.closed_form(q, k, v, lengths=end, k_scale=ks, v_scale=vs)
+  gq, gk, gv, gks, gvs, gend = to_dev(q, k, v, ks, vs, end)
+  o, (m, l) = ak.ragged_mha(gq, gk, gv, 0, None, gend, None, None, gks, gvs)
+  check_out(o.reshape(b, hq, 1, d), wo, "very large batch")
+  check_stats(m, l, wm, wl, (end > 0).reshape(b, 1, 1, 1).expand(b, hq, 1, 1))
+
+
 def test_ragged_stacked_cache_selects_layer_and_reuses_plan():
   from jetstream_pt_amd import attention_kernel as ak
   g = torch.Generator().manual_seed(301)
