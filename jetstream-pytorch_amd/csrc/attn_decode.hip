@@ -82,6 +82,30 @@ Layout make_layout(int batch, int kv_heads, int rows) {
 // (an empty slot still needs one item per head to write its output);
 // entries are counting-sorted by tile count, longest first; records past the
 // last entry are marked unused.
+// Exclusive prefix sum of `x` over the 256 threads of the planning workgroup;
+// *total gets the sum.
+__device__ __forceinline__ int plan_exclusive_scan(int x, int* total) {
+  __shared__ int s_wave[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int incl = x;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int y = __shfl_up(incl, off);
+    if (lane >= off) incl += y;
+  }
+  __syncthreads();  // s_wave may still be read from the previous call
+  if (lane == 63) s_wave[wave] = incl;
+  __syncthreads();
+  int before = 0, sum = 0;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    if (w < wave) before += s_wave[w];
+    sum += s_wave[w];
+  }
+  *total = sum;
+  return before + incl - x;
+}
+
 __global__ void __launch_bounds__(256)
 plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int target,
             PlanEntry* entries, SlotChunks* slots, int max_entries) {
@@ -110,16 +134,23 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     c = c < floor_c ? floor_c : c;  // at most kMaxChunksPerSlot chunks per slot
     c = (c + kChunkAlign - 1) / kChunkAlign * kChunkAlign;
     s_chunk = c < kChunkAlign ? kChunkAlign : static_cast<int>(c);
-    int first = 0;
-    for (int b = 0; b < batch; ++b) {  // LDS only: a few cycles per slot
-      s_first[b] = first;
-      first += s_len[b] == 0 ? 1 : (s_len[b] + s_chunk - 1) / s_chunk;
-    }
-    s_entries = first;
   }
   __syncthreads();
   const int chunk = s_chunk;
   auto chunks_of = [&](int b) { return s_len[b] == 0 ? 1 : (s_len[b] + chunk - 1) / chunk; };
+  // a slot's first partial record: running sum of the chunk counts, 256 slots a pass
+  {
+    int base = 0;
+    for (int b0 = 0; b0 < batch; b0 += static_cast<int>(blockDim.x)) {
+      const int b = b0 + tid;
+      int total;
+      const int before = plan_exclusive_scan(b < batch ? chunks_of(b) : 0, &total);
+      if (b < batch) s_first[b] = base + before;
+      base += total;
+    }
+    if (tid == 0) s_entries = base;
+  }
+  __syncthreads();
   auto key_of = [&](int count) {
     const int tiles = (count + kTile - 1) / kTile;
     return tiles > 256 ? 256 : tiles;
@@ -130,12 +161,12 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     for (int c = 0; c < nc; ++c) atomicAdd(&s_hist[key_of(min(chunk, s_len[b] - c * chunk))], 1);
   }
   __syncthreads();
-  if (tid == 0) {
-    int run = 0;
-    for (int k = 256; k >= 0; --k) {
-      s_base[k] = run;
-      run += s_hist[k];
-    }
+  {
+    // where each tile count's entries start, longest first: thread t has key 256 - t
+    int total;
+    const int before = plan_exclusive_scan(s_hist[256 - tid], &total);
+    s_base[256 - tid] = before;
+    if (tid == 0) s_base[0] = total;
   }
   __syncthreads();
   for (int b = tid; b < batch; b += blockDim.x) {

@@ -64,66 +64,102 @@ dpam_init_kernel(jpt_dpam d, const int32_t* free_order) {
   }
 }
 
-// reserve_pages_insert (:42-52), requests served one after another.
+// reserve_pages_insert (:42-52), requests served one after another.  The free
+// list's head and count travel in registers (every thread computes the same
+// values) and the requests are read kThreads at a time, so a request costs one
+// memory round trip - ring to table row - and no barrier: rows and ring cells
+// of different requests are disjoint, and a slot named twice is written twice
+// by the same threads in request order.
 __global__ void __launch_bounds__(kThreads)
 dpam_reserve_insert_kernel(jpt_dpam d, const int32_t* slots, const int32_t* seq_lens, int n_req,
                            int slot_imm, int len_imm) {
-  for (int r = 0; r < n_req; ++r) {
-    const int slot = slots ? slots[r] : slot_imm;
-    const int len = seq_lens ? seq_lens[r] : len_imm;
-    const int head = d.state[0], count = d.state[1];
-    __syncthreads();  // everyone has read the state before thread 0 moves it
-    if (slot < 0 || slot >= d.batch || len < 0) {
-      if (threadIdx.x == 0) raise(d, JPT_DPAM_BADARG);
-      continue;
+  __shared__ int s_slot[kThreads], s_len[kThreads];
+  int head = d.state[0], count = d.state[1];
+  for (int r0 = 0; r0 < n_req; r0 += kThreads) {
+    __syncthreads();  // the previous batch of requests has been read
+    if (r0 + threadIdx.x < n_req) {
+      s_slot[threadIdx.x] = slots ? slots[r0 + threadIdx.x] : slot_imm;
+      s_len[threadIdx.x] = seq_lens ? seq_lens[r0 + threadIdx.x] : len_imm;
     }
-    const int n = (len + d.page_size - 1) / d.page_size;
-    if (n > d.max_pages) {
-      if (threadIdx.x == 0) raise(d, JPT_DPAM_OVERFLOW);
-      continue;
+    __syncthreads();
+    const int n_here = min(kThreads, n_req - r0);
+    for (int j = 0; j < n_here; ++j) {
+      const int slot = s_slot[j], len = s_len[j];
+      if (slot < 0 || slot >= d.batch || len < 0) {
+        if (threadIdx.x == 0) raise(d, JPT_DPAM_BADARG);
+        continue;
+      }
+      const int n = (len + d.page_size - 1) / d.page_size;
+      if (n > d.max_pages) {
+        if (threadIdx.x == 0) raise(d, JPT_DPAM_OVERFLOW);
+        continue;
+      }
+      if (n > count) {
+        if (threadIdx.x == 0) raise(d, JPT_DPAM_NOPAGES);
+        continue;
+      }
+      int32_t* row = d.page_indices + static_cast<int64_t>(slot) * d.max_pages;
+      for (int i = threadIdx.x; i < n; i += kThreads) row[i] = d.ring[(head + i) % d.total_pages];
+      if (threadIdx.x == 0) {
+        d.lengths[slot] = len;
+        d.n_alloc[slot] = n;
+      }
+      head = (head + n) % d.total_pages;
+      count -= n;
     }
-    if (n > count) {
-      if (threadIdx.x == 0) raise(d, JPT_DPAM_NOPAGES);
-      continue;
-    }
-    int32_t* row = d.page_indices + static_cast<int64_t>(slot) * d.max_pages;
-    for (int i = threadIdx.x; i < n; i += kThreads) row[i] = d.ring[(head + i) % d.total_pages];
-    if (threadIdx.x == 0) {
-      d.state[0] = (head + n) % d.total_pages;
-      d.state[1] = count - n;
-      d.lengths[slot] = len;
-      d.n_alloc[slot] = n;
-    }
-    __syncthreads();  // the next request sees the moved state
+  }
+  if (threadIdx.x == 0) {
+    d.state[0] = head;
+    d.state[1] = count;
   }
 }
 
 // free_pages_resource (:214-222): the slot's pages go to the tail of the free
-// list in row order; row back to the sentinel, length to 0.
+// list in row order; row back to the sentinel, length to 0.  Requests are read
+// kThreads at a time together with their slots' page counts; a slot named
+// again later in the list has nothing left to free by then.
 __global__ void __launch_bounds__(kThreads)
 dpam_free_kernel(jpt_dpam d, const int32_t* slots, int n_req, int slot_imm) {
-  for (int r = 0; r < n_req; ++r) {
-    const int slot = slots ? slots[r] : slot_imm;
-    const int head = d.state[0], count = d.state[1];
-    __syncthreads();
-    if (slot < 0 || slot >= d.batch) {
-      if (threadIdx.x == 0) raise(d, JPT_DPAM_BADARG);
-      continue;
+  __shared__ int s_slot[kThreads], s_n[kThreads];
+  const int head = d.state[0];
+  int count = d.state[1];
+  for (int r0 = 0; r0 < n_req; r0 += kThreads) {
+    __syncthreads();  // the previous batch is done, its page counts are written
+    const int n_here = min(kThreads, n_req - r0);
+    int slot = -1, n = 0;
+    if (static_cast<int>(threadIdx.x) < n_here) {
+      slot = slots ? slots[r0 + threadIdx.x] : slot_imm;
+      if (slot >= 0 && slot < d.batch) n = d.n_alloc[slot];
     }
-    int32_t* row = d.page_indices + static_cast<int64_t>(slot) * d.max_pages;
-    int n = d.n_alloc[slot];
-    n = min(max(n, 0), min(d.max_pages, d.total_pages - count));  // never more than the ring has room for
-    const int tail = (head + count) % d.total_pages;
-    for (int i = threadIdx.x; i < n; i += kThreads) d.ring[(tail + i) % d.total_pages] = row[i];
-    __syncthreads();  // rows are read before they are reset
-    for (int i = threadIdx.x; i < d.max_pages; i += kThreads) row[i] = d.total_pages - 1;
-    if (threadIdx.x == 0) {
-      d.state[1] = count + n;
-      d.n_alloc[slot] = 0;
-      d.lengths[slot] = 0;
-    }
+    s_slot[threadIdx.x] = slot;
     __syncthreads();
+    for (int j = 0; j < static_cast<int>(threadIdx.x) && j < n_here; ++j)
+      if (s_slot[j] == slot) n = 0;
+    s_n[threadIdx.x] = n;
+    __syncthreads();
+    for (int j = 0; j < n_here; ++j) {
+      const int sl = s_slot[j];
+      if (sl < 0 || sl >= d.batch) {
+        if (threadIdx.x == 0) raise(d, JPT_DPAM_BADARG);
+        continue;
+      }
+      int32_t* row = d.page_indices + static_cast<int64_t>(sl) * d.max_pages;
+      // never more than the ring has room for
+      const int m = min(max(s_n[j], 0), min(d.max_pages, d.total_pages - count));
+      const int tail = (head + count) % d.total_pages;
+      // a thread reads the cells it resets: no barrier between the two
+      for (int i = threadIdx.x; i < d.max_pages; i += kThreads) {
+        if (i < m) d.ring[(tail + i) % d.total_pages] = row[i];
+        row[i] = d.total_pages - 1;
+      }
+      if (threadIdx.x == 0) {
+        d.n_alloc[sl] = 0;
+        d.lengths[sl] = 0;
+      }
+      count += m;
+    }
   }
+  if (threadIdx.x == 0) d.state[1] = count;
 }
 
 // fill_new_pages (:55-64) followed by get_page_token_indices (:145-177) on the
