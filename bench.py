@@ -22,8 +22,8 @@ c1|c2|c4|c5` times them the same way for the record (same JSON shape, no
 cpu_baseline):
   c1  dense bf16 eager update + dense attention, B=8, 32 heads, S=1024
   c2  int8 MHA decode step, B=96, 32 heads, S=2048, lengths U[128, 2048]
-  c4  paged bf16, B=256, 64 q / 8 kv heads, 32768 pages of 64, host page
-      allocation every decode step, paged append + paged attention
+  c4  paged bf16, B=256, 64 q / 8 kv heads, 32768 pages of 64, page
+      allocation every decode step, paged attention that appends the token
   c5  paged int8, 32 layers, B=256, 32 q / 8 kv heads, 16384 pages of 64 per
       layer; every decode step frees 16 slots and inserts 16 new prompts
 """
@@ -211,7 +211,8 @@ def build_c1(torch, args):
 
 def build_paged(torch, args, int8):
   """c4 (bf16 pages) / c5 (int8 pages, prompt churn): page allocation once per
-  decode step, then per layer a paged append and a paged attention.  By default
+  decode step, then per layer a paged append and a paged attention (one launch
+  with the device allocator: the attention launch appends the token).  By default
   the allocator, its tables and the per-slot lengths live on the device and a
   decode step is replayed from one HIP graph (allocation, token indices, all
   layers, position advance); prompt churn is enqueued between replays.
@@ -357,9 +358,10 @@ def build_paged(torch, args, int8):
 
   where = "host page allocation (lengths pulled, tables uploaded)" if host_alloc else \
       "page allocation, token indices and position advance on the device"
+  per_layer = "paged append + paged attention" if host_alloc else "one paged attention launch that also appends the token"
   name = ("C5 paged int8 layer-step: per decode step 16 slots freed and 16 prompts quantised into pages (all "
-          f"layers), {where}; per layer quantised paged append + paged attention" if int8 else
-          f"C4 paged bf16 layer-step: {where} once per decode step; per layer paged append + paged attention")
+          f"layers), {where}; per layer {'quantised ' if host_alloc else ''}{per_layer}" if int8 else
+          f"C4 paged bf16 layer-step: {where} once per decode step; per layer {per_layer}")
   return dict(step=step, before_pass=before_pass, attn_only=attn_only, bytes_now=bytes_now, graph=not host_alloc,
               pam=pam, pools=(pools_k, pools_v), dlens=dlens,
               scale_pages=(sk, sv), caches=caches, state=state, xq=xq, xk=xk, xv=xv, env=env,

@@ -271,6 +271,18 @@ int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void* stream);
  * attended with them.  One launch less per layer; the reference has the
  * quantiser and the attention as separate XLA ops.
  *
+ * new_to_pages (jpt_attn_paged only): the call also does the work of
+ * jpt_paged_append / jpt_paged_append_quant_i8 for the new token
+ * (PageKVCacheGenerate.update, cache_manager.py:663-724): `lengths` are the
+ * slots' lengths BEFORE the step; the token of slot b is attended and written
+ * to position lengths[b] of the slot - page page_table[b][lengths[b] /
+ * page_size], whose id the allocator has already put there - codes (or bf16
+ * rows) into k/v, scales into k_scale/v_scale, which become outputs for those
+ * rows.  A slot of length 0 is inactive, as in the reference's token indices
+ * (page_attention_manager.py:145-177): nothing is written or attended for it.
+ * Needs the streaming kernel's shapes (dim 128, bf16 query, page_size a
+ * multiple of 32); other shapes are refused.
+ *
  * workspace: device scratch of at least jpt_attn_workspace_bytes(args)
  * bytes, 256-byte aligned.  Its first JPT_ATTN_WS_STATE_BYTES must be zero
  * before the first call and are left zero by every call; calls sharing one
@@ -315,6 +327,7 @@ typedef struct {
   const float* new_k_rope; /* NULL, or rotary factors (batch, dim / 2, 2) as in
                               jpt_quant_append_args: new_k_raw is unrotated and is
                               rotated before it is quantised (needs new_k_raw) */
+  int32_t new_to_pages;    /* see above */
 } jpt_attn_args;
 
 int64_t jpt_attn_workspace_bytes(const jpt_attn_args* args);

@@ -174,11 +174,11 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     for (int c = 0; c < nc; ++c) {
       const int count = min(chunk, s_len[b] - c * chunk);
       const int at = atomicAdd(&s_base[key_of(count)], 1);
-      if (at < max_entries) entries[at] = PlanEntry{b, c * chunk, count, first + c, nc, {0, 0, 0}};
+      if (at < max_entries) entries[at] = PlanEntry{b, c * chunk, count, first + c, nc, s_len[b], {0, 0}};
     }
   }
   for (int i = s_entries + tid; i < max_entries; i += blockDim.x)
-    entries[i] = PlanEntry{-1, 0, 0, 0, 0, {0, 0, 0}};
+    entries[i] = PlanEntry{-1, 0, 0, 0, 0, 0, {0, 0}};
 }
 
 // Folds the partials of every slot that was split into several chunks: one
@@ -368,6 +368,7 @@ static int32_t attn_entry(const jpt_attn_args* args, jpt::AttnMode mode, void* s
     a.new_k_rope = nullptr;
     if (attn_fast_supported(a, mode)) return attn_fast_launch(a, mode, s);
   }
+  JPT_REQUIRE(!a.new_to_pages, "new_to_pages needs head_dim 128, a bf16 query and page_size a multiple of 32");
   return attn_generic_launch(a, mode, s);
 }
 

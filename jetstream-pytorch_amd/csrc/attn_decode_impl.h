@@ -313,6 +313,7 @@ struct Tile<__bf16> {
 // One work item: a chunk of one slot for one KV head.
 struct Item {
   int slot, start, count, part, n_chunks, h;
+  int len;  // positions of the whole slot
   bool valid;
 };
 
@@ -365,6 +366,8 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   const bool has_new = a.new_k != nullptr;
   // the new token arrives unquantised: the consumer of its tile quantises it
   const bool quant_new = std::is_same<KV, int8_t>::value && a.new_k_raw != nullptr;
+  // the new token is also written into its slot's page (paged caches)
+  const bool to_pages = PAGED && has_new && a.new_to_pages != 0;
 
   // Item of round k of this worker: virtual ids k*G + j with j running forwards
   // in even rounds and backwards in odd ones, so that with entries sorted
@@ -404,9 +407,9 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       e0 = en[0];
       e1 = en[1];
     }
-    // slot, start, count, part | n_chunks, head, valid
+    // slot, start, count, part | n_chunks, head, valid, slot length
     *reinterpret_cast<int4*>(&sm_items[lane][0]) = e0;
-    *reinterpret_cast<int4*>(&sm_items[lane][4]) = make_int4(e1.x, h, e0.x >= 0 ? 1 : 0, 0);
+    *reinterpret_cast<int4*>(&sm_items[lane][4]) = make_int4(e1.x, h, e0.x >= 0 ? 1 : 0, e1.y);
   }
   __syncthreads();
   auto unpack_item = [&](int4 e0, int4 e1) -> Item {
@@ -418,27 +421,29 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     it.n_chunks = __builtin_amdgcn_readfirstlane(e1.x);
     it.h = __builtin_amdgcn_readfirstlane(e1.y);
     it.valid = __builtin_amdgcn_readfirstlane(e1.z) != 0;
+    it.len = __builtin_amdgcn_readfirstlane(e1.w);
     return it;
   };
   auto fetch = [&](int k) -> Item {  // rounds past the listed ones
     Item it;
     int entry, h;
     it.valid = item_index(k, &entry, &h);
-    it.slot = it.start = it.count = it.part = it.n_chunks = it.h = 0;
+    it.slot = it.start = it.count = it.part = it.n_chunks = it.h = it.len = 0;
     if (it.valid) {
       const int32_t* en = reinterpret_cast<const int32_t*>(p.entries + entry);
       it.h = h;
       it.slot = load_uniform(en + 0); it.start = load_uniform(en + 1); it.count = load_uniform(en + 2);
-      it.part = load_uniform(en + 3); it.n_chunks = load_uniform(en + 4);
+      it.part = load_uniform(en + 3); it.n_chunks = load_uniform(en + 4); it.len = load_uniform(en + 5);
       it.valid = it.slot >= 0;
     }
     return it;
   };
   // tiles of an item: its cache positions, plus one for the step's new token
-  // on the slot's first chunk
+  // on the slot's first chunk (when the token also goes into the pages, an
+  // empty slot is an inactive one and has no token)
   auto cache_tiles = [&](const Item& it) { return (it.count + kTile - 1) / kTile; };
   auto item_tiles = [&](const Item& it) {
-    return cache_tiles(it) + ((has_new && it.start == 0) ? 1 : 0);
+    return cache_tiles(it) + ((has_new && it.start == 0 && !(to_pages && it.len == 0)) ? 1 : 0);
   };
   // Bounded wait for an LDS counter; false = give up (abort raised).
   auto wait_for = [&](int* counter, int needed) -> bool {
@@ -841,6 +846,13 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     }
     return sc;
   };
+  // The new token on its way into the slot's page (to_pages): the lane's bytes of
+  // its key and value rows and its scales, kept from its tile until the item's
+  // other tiles are done, when the page id asked for at the item's start is there.
+  constexpr int kLaneBytes = C::kRowBytes / 64;  // 2 (codes) or 4 (bf16)
+  uint32_t keep_k = 0, keep_v = 0;
+  float keep_ks = 0.f, keep_vs = 0.f;
+  bool keep = false;
   auto consume_tile = [&](int t, int valid, bool is_new, auto full_tag) -> bool {
     constexpr bool FULL = decltype(full_tag)::value;
     const int s = t % C::kSlots;
@@ -905,6 +917,20 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
 #pragma unroll
         for (int i = 0; i < 8; ++i) mk[i] = 0.f;
       }
+    }
+    if (!FULL && is_new && to_pages) {  // row 0 of the tile: piece p sits at piece slot p
+      if (kLaneBytes == 2) {
+        keep_k = *reinterpret_cast<const uint16_t*>(slot + lane * 2);
+        keep_v = *reinterpret_cast<const uint16_t*>(slot + C::kTileBytes + lane * 2);
+      } else {
+        keep_k = *reinterpret_cast<const uint32_t*>(slot + lane * 4);
+        keep_v = *reinterpret_cast<const uint32_t*>(slot + C::kTileBytes + lane * 4);
+      }
+      if (SCALE) {
+        keep_ks = ks[0];
+        keep_vs = vs[0];
+      }
+      keep = true;
     }
     // the registers hold the tile: hand the slot back (the release waits for
     // the LDS reads above)
@@ -1130,6 +1156,12 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     }
     cur_slot = cur.slot;
     cur_h = cur.h;
+    // where the new token goes: the page of position cur.len (asked for now, used
+    // after the item's tiles)
+    int dst_page = 0;
+    const bool dst_room = cur.len < a.max_pages * a.page_size;
+    if (to_pages && cur.start == 0 && cur.len > 0 && dst_room)
+      dst_page = a.page_table[static_cast<int64_t>(cur.slot) * a.max_pages + cur.len / a.page_size];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
     accw = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -1143,6 +1175,28 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         if (!consume_tile(base + ti, valid, false, std::true_type{})) return;
       } else {
         if (!consume_tile(base + ti, valid, is_new, std::false_type{})) return;
+      }
+    }
+    if (keep) {  // this consumer had the new token's tile
+      keep = false;
+      if (dst_room) {
+        const int page = min(max(dst_page, 0), a.total_pages - 1);  // whatever the table holds, stay inside the pool
+        const int64_t in_pool = static_cast<int64_t>(page) * a.page_size + cur.len % a.page_size;
+        const int64_t row = static_cast<int64_t>(cur.h) * a.total_pages * a.page_size + in_pool;
+        char* dk = static_cast<char*>(const_cast<void*>(a.k)) + row * C::kRowBytes + lane * kLaneBytes;
+        char* dv = static_cast<char*>(const_cast<void*>(a.v)) + row * C::kRowBytes + lane * kLaneBytes;
+        if (kLaneBytes == 2) {
+          *reinterpret_cast<uint16_t*>(dk) = static_cast<uint16_t>(keep_k);
+          *reinterpret_cast<uint16_t*>(dv) = static_cast<uint16_t>(keep_v);
+        } else {
+          *reinterpret_cast<uint32_t*>(dk) = keep_k;
+          *reinterpret_cast<uint32_t*>(dv) = keep_v;
+        }
+        if (SCALE && lane == 0 && (a.scale_heads != 1 || cur.h == 0)) {
+          const int64_t si = static_cast<int64_t>(a.scale_heads == 1 ? 0 : cur.h) * a.total_pages * a.page_size + in_pool;
+          store_from_f32(const_cast<void*>(a.k_scale), si, kBf16Math ? JPT_BF16 : JPT_F32, keep_ks);
+          store_from_f32(const_cast<void*>(a.v_scale), si, kBf16Math ? JPT_BF16 : JPT_F32, keep_vs);
+        }
       }
     }
     JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)

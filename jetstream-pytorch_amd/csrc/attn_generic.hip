@@ -208,7 +208,9 @@ int32_t check_attn_args(const jpt_attn_args& a, AttnMode mode) {
     JPT_REQUIRE(a.page_table && a.lengths, "paged attention needs page_table and lengths");
     JPT_REQUIRE(a.total_pages > 0 && a.page_size > 0 && a.max_pages > 0, "total_pages, page_size, max_pages must be positive");
     JPT_REQUIRE(a.mask == nullptr, "paged attention takes no mask");
+    JPT_REQUIRE(!a.new_to_pages || a.new_k != nullptr, "new_to_pages needs the new token (new_k/new_v)");
   } else {
+    JPT_REQUIRE(!a.new_to_pages, "new_to_pages is for the paged entry point");
     JPT_REQUIRE(a.seq > 0, "seq must be positive");
     JPT_REQUIRE(a.page_table == nullptr, "page_table given to a non-paged entry point");
     if (mode == kRagged) JPT_REQUIRE(a.lengths != nullptr, "ragged attention needs lengths");

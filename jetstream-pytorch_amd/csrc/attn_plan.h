@@ -17,7 +17,8 @@ struct PlanEntry {
   int32_t count;       // positions in the chunk (0 for an empty slot)
   int32_t part;        // index of this chunk's partial record
   int32_t n_chunks;    // chunks of this slot
-  int32_t pad[3];
+  int32_t slot_len;    // positions of the whole slot
+  int32_t pad[2];
 };
 struct SlotChunks {
   int32_t n_chunks, first_part;

@@ -97,7 +97,7 @@ class AttnArgs(_c.Structure):
       ("scale_dtype", _i32), ("scale_heads", _i32), ("mask_dtype", _i32),
       ("sm_scale", _f32), ("force_generic", _i32), ("reuse_plan", _i32),
       ("new_k_raw", _vp), ("new_v_raw", _vp), ("new_rounding", _i32),
-      ("new_k_rope", _vp),
+      ("new_k_rope", _vp), ("new_to_pages", _i32),
   ]
 
 

@@ -129,8 +129,8 @@ def _scale_tensor(s, paged):
 def _attend(mode, xq, keys, values, *, lengths=None, page_table=None, mask=None,
             k_scaler=None, v_scaler=None, sm_scale=None, new_key=None,
             new_value=None, new_k_scaler=None, new_v_scaler=None, new_key_raw=None,
-            new_value_raw=None, new_rounding="trunc", new_key_rope=None, want_stats=False,
-            plan=None, force_generic=False):
+            new_value_raw=None, new_rounding="trunc", new_key_rope=None, new_to_pages=False,
+            want_stats=False, plan=None, force_generic=False):
   """xq (B, Hq, T, D); keys/values (B, Hkv, S, D) or pages (Hkv, P, ps, D).
   Returns (o (B, Hq, T, D), max (B, Hq, T) | None, denom (B, Hq, T) | None)."""
   xq = _ffi.dev(xq, "xq")
@@ -219,6 +219,10 @@ def _attend(mode, xq, keys, values, *, lengths=None, page_table=None, mask=None,
         keep.append(rope)
     elif new_key_rope is not None:
       raise ValueError("new_key_rope goes with new_key_raw (the launch that quantises the token rotates it)")
+  if new_to_pages:
+    if mode != "paged" or new_key is None:
+      raise ValueError("new_to_pages goes with paged attention and a new token")
+    a.new_to_pages = 1
   a.sm_scale = 1.0 / math.sqrt(d) if sm_scale is None else float(sm_scale)
   a.force_generic = int(force_generic)
 
@@ -352,19 +356,28 @@ class RaggedAttentionKernel:
 
 
 def call_paged_attention(env, xq, keys, values, seq_lens, page_indices, *, sm_scale=1.0,
-                         k_scaler=None, v_scaler=None, plan=None):
+                         k_scaler=None, v_scaler=None, plan=None, append=None):
   """Paged decode attention: xq (B, Hq, D), pages (Hkv, P, ps, D), seq_lens
   (B,), page_indices (B, max_pages); returns (B, Hq, D).  seq_lens and
   page_indices may be numpy arrays (as PageAttentionManager holds them) or
-  int32 device tensors.  With int8 pages pass scale pages (Hs, P, ps)."""
+  int32 device tensors.  With int8 pages pass scale pages (Hs, P, ps).
+
+  append: None, or the step's own token as a dict of the new-token keywords of
+  ragged_mha (new_key/new_value in the pages' dtype with their scalers, or
+  new_key_raw/new_value_raw bf16 plus output tensors).  The launch then also
+  appends the token to the pages (PageKVCacheGenerate.update's scatter,
+  cache_manager.py:663-724) and attends it: seq_lens are the lengths BEFORE the
+  step, slots of length 0 are inactive, and the page of position seq_lens[b]
+  must already be in page_indices."""
   del env
   device = xq.device
   if not isinstance(page_indices, torch.Tensor):
     import numpy as np
     page_indices = torch.from_numpy(np.ascontiguousarray(page_indices, dtype=np.int32)).to(device)
+  extra = {} if append is None else dict(append, new_to_pages=True)
   out, _, _ = _attend("paged", xq.unsqueeze(2), keys, values, lengths=seq_lens,
                       page_table=page_indices, k_scaler=k_scaler, v_scaler=v_scaler,
-                      sm_scale=sm_scale, plan=plan)
+                      sm_scale=sm_scale, plan=plan, **extra)
   return out.squeeze(2)
 
 

@@ -352,8 +352,11 @@ class PageKVCacheGenerate:
     self.env = env
     self.stacked = False
 
-  def update(self, key, value, layer_id=0):
-    """Update kv cache"""
+  def update(self, key, value, layer_id=0, *, defer_append=False):
+    """Update kv cache.  defer_append: write nothing - the attention launch
+    appends the token itself (call_paged_attention(append=...))."""
+    if defer_append:
+      return self.cache_k, self.cache_v
     pk, pv = _ffi.dev(self.cache_k, "cache_k"), _ffi.dev(self.cache_v, "cache_v")
     heads, total, ps, dim = pk.shape
     key = _ffi.dev(key.to(pk.dtype).contiguous(), "key")
@@ -407,8 +410,12 @@ class Int8PageKVCacheGenerate:
     self.stacked = False
     self.rounding = rounding
 
-  def update(self, key, value, layer_id=0, *, freqs_cis=None):
-    """freqs_cis: rotary factors of the step when `key` is still unrotated."""
+  def update(self, key, value, layer_id=0, *, freqs_cis=None, defer_append=False):
+    """freqs_cis: rotary factors of the step when `key` is still unrotated.
+    defer_append: write nothing - the attention launch quantises and appends
+    the token itself (call_paged_attention(append=...))."""
+    if defer_append:
+      return self.cache_k, self.cache_v, self.k_scaler, self.v_scaler
     pk, pv = _ffi.dev(self.cache_k, "cache_k"), _ffi.dev(self.cache_v, "cache_v")
     ks, vs = _ffi.dev(self.k_scaler, "k_scale_pages"), _ffi.dev(self.v_scaler, "v_scale_pages")
     heads, total, ps, dim = pk.shape

@@ -73,12 +73,15 @@ class AttentionKernel:
     elif env.page_attention and seqlen == 1 and hasattr(cache, "page_attention_manager"):
       pam = cache.page_attention_manager
       lengths, page_indices = pam.device_tables(xq.device)
+      if new_token is not None:  # the launch appends the token: lengths before the step
+        lengths = pam.step_lens
       # one split plan per decode step, shared by the layers
       plan = ak.paged_decode_plan(pam, lengths, bsz, num_heads, keys.shape[0], keys.shape[2],
                                   page_indices.shape[1])
       local_output = self.page_attention(
           env, torch.squeeze(xq, 2), keys, values, lengths, page_indices,
-          sm_scale=self.sm_scale_paged, k_scaler=k_scaler, v_scaler=v_scaler, plan=plan)
+          sm_scale=self.sm_scale_paged, k_scaler=k_scaler, v_scaler=v_scaler, plan=plan,
+          append=new_token)
     else:
       local_output = self.dense_attention(
           xq=xq, keys=keys, values=values, k_scaler=k_scaler, v_scaler=v_scaler, mask=local_mask)
@@ -87,6 +90,16 @@ class AttentionKernel:
       local_max = local_max.reshape(bsz, num_heads, seqlen, 1)
       local_denom = local_denom.reshape(bsz, num_heads, seqlen, 1)
     return local_output, (local_max, local_denom)
+
+  def _will_append_in_launch(self, xq, cache, keys):
+    """Paged cache, one token per slot, the device-resident allocator (its
+    lengths before the step stay on the device) and the streaming kernel's
+    shapes: the attention launch appends the step's token to the pages itself."""
+    pam = getattr(cache, "page_attention_manager", None)
+    return (self.fuse_new_token and self.env.page_attention and xq.shape[2] == 1
+            and getattr(pam, "step_lens", None) is not None and xq.dtype == torch.bfloat16
+            and xq.shape[3] == 128 and keys.dim() == 4 and keys.shape[2] % 32 == 0
+            and not (self.env.ragged_mha or self.env.flash_attention))
 
   def _will_fuse(self, seqlen, keys):
     env = self.env
@@ -98,8 +111,12 @@ class AttentionKernel:
     """xq (batch, heads, seqlen, head_dim); xk, xv (batch, kv_heads, seqlen, head_dim);
     mask additive 0/-inf or None; cache a CacheInterface object."""
     seqlen = xq.shape[2]
-    orig_keys, orig_values = cache.update(xk, xv, self.layer_id)
     args = (cache, start, end, ragged_batch_index, ragged_block_index)
+    if hasattr(cache, "page_attention_manager") and self._will_append_in_launch(xq, cache, cache.cache_k):
+      keys, values = cache.update(xk, xv, self.layer_id, defer_append=True)
+      new = dict(new_key=xk.to(keys.dtype).contiguous(), new_value=xv.to(keys.dtype).contiguous())
+      return self._attend(xq, keys, values, None, None, mask, *args, new_token=new)[0]
+    orig_keys, orig_values = cache.update(xk, xv, self.layer_id)
     if self._will_fuse(seqlen, orig_keys):
       dt = orig_keys.dtype
       new = dict(new_key=xk.to(dt).contiguous(), new_value=xv.to(dt).contiguous())
@@ -130,6 +147,21 @@ class Int8KVAttentionKernel(AttentionKernel):
       xk = apply_rotary_emb(None, xk.transpose(1, 2), freqs_cis)[1].transpose(1, 2)
       freqs_cis = None
     rope_kw = {} if freqs_cis is None else {"freqs_cis": freqs_cis}
+    args = (cache, start, end, ragged_batch_index, ragged_block_index)
+    if (hasattr(cache, "page_attention_manager") and hasattr(cache, "rounding")
+        and self._will_append_in_launch(xq, cache, cache.cache_k) and xk.dtype == torch.bfloat16):
+      # int8 pages: the attention launch quantises the token, writes codes and
+      # scales into its page and attends it
+      keys, values, k_scaler, v_scaler = cache.update(xk, xv, self.layer_id, defer_append=True)
+      bsz, hkv, _, dim = xk.shape
+      hs = k_scaler.shape[0]
+      new = dict(new_key=torch.empty((bsz, hkv, 1, dim), dtype=torch.int8, device=xk.device),
+                 new_value=torch.empty((bsz, hkv, 1, dim), dtype=torch.int8, device=xk.device),
+                 new_k_scaler=torch.empty((bsz, hs), dtype=k_scaler.dtype, device=xk.device),
+                 new_v_scaler=torch.empty((bsz, hs), dtype=k_scaler.dtype, device=xk.device),
+                 new_key_raw=xk.contiguous(), new_value_raw=xv.contiguous(), new_rounding=cache.rounding,
+                 new_key_rope=freqs_cis)
+      return self._attend(xq, keys, values, k_scaler, v_scaler, mask, *args, new_token=new)[0]
     # the ragged launch can quantise the token itself (one launch less)
     fuse_quant = (self.fuse_quantize and isinstance(cache, Int8KVCacheGenerate)
                   and self._will_fuse(seqlen, cache.cache_k) and xk.dtype == torch.bfloat16
@@ -142,7 +174,6 @@ class Int8KVAttentionKernel(AttentionKernel):
     else:
       (orig_keys, orig_values, new_key, new_value, k_scaler, v_scaler, new_k_scaler,
        new_v_scaler) = ret
-    args = (cache, start, end, ragged_batch_index, ragged_block_index)
     if new_key is not None and self._will_fuse(seqlen, orig_keys):
       new = dict(new_key=new_key, new_value=new_value, new_k_scaler=new_k_scaler,
                  new_v_scaler=new_v_scaler)

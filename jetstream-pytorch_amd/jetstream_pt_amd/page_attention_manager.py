@@ -241,6 +241,7 @@ class DevicePageAttentionManager(PageAttentionManager):
     self._keep = order  # read by the enqueued kernel
     self._token_indices = DeviceTokenIndices(self._update_indices, self._state[3:4])
     self._stepped = False
+    self.step_lens = None
     self._version = 1  # bumped by every launch that changes `lengths`
 
   def __del__(self):
@@ -290,6 +291,9 @@ class DevicePageAttentionManager(PageAttentionManager):
     _ffi.check(_ffi.lib.jpt_dpam_decode_step(self._c, _ffi.ptr(lens), _ffi.stream()))
     self._stepped = True
     self._version += 1
+    # the lengths before the step's token, for an attention launch that appends
+    # the token itself; valid until the caller advances `lens`
+    self.step_lens = lens
 
   # pylint: disable-next=all
   def get_page_token_indices(self, lens):

@@ -200,15 +200,21 @@ def _paged_setup(int8, seed):
   return env, hp, dp, caches, lens, (b, hq, hkv, d), g
 
 
+@pytest.mark.parametrize("fused", [False, True])
 @pytest.mark.parametrize("int8", [False, True])
-def test_paged_decode_steps_device_allocator_equals_host_allocator(int8):
+def test_paged_decode_steps_device_allocator_equals_host_allocator(int8, fused):
   """Whole decode steps - page allocation, token indices, (quantised) paged
   append, paged attention, position advance - with nothing crossing to the
-  host, eagerly and as replays of one captured HIP graph; pages, scale pages,
-  tables and outputs must equal the host-allocator flow bit for bit."""
+  host, eagerly and as replays of one captured HIP graph; pages, scale pages
+  and tables must equal the host-allocator flow bit for bit.  fused: the
+  device flow's attention launch appends (and quantises) the token itself - no
+  append launch; its outputs sum in another order, so they are held to the
+  attention tolerance instead of bit equality."""
   from jetstream_pt_amd import decode_state, layers
   env, hp, dp, (hc, dc), lens, (b, hq, hkv, d), g = _paged_setup(int8, 401 + int(int8))
-  kern = (layers.Int8KVAttentionKernel if int8 else layers.AttentionKernel)(env, 0)
+  cls = layers.Int8KVAttentionKernel if int8 else layers.AttentionKernel
+  kern_h = cls(env, 0, fuse_new_token=False)
+  kern = cls(env, 0, fuse_new_token=fused)
   dlens = torch.from_numpy(lens).to(DEV)
   xq = torch.empty((b, hq, 1, d), dtype=torch.bfloat16, device=DEV)
   xk = torch.empty((b, hkv, 1, d), dtype=torch.bfloat16, device=DEV)
@@ -217,6 +223,7 @@ def test_paged_decode_steps_device_allocator_equals_host_allocator(int8):
 
   def device_step():
     dc.page_token_indices = dp.decode_step(dlens)
+    assert kern._will_append_in_launch(xq, dc, dc.cache_k) == fused
     out_d.copy_(kern(xq, xk, xv, None, dc))
     decode_state.advance(dlens)
 
@@ -224,9 +231,17 @@ def test_paged_decode_steps_device_allocator_equals_host_allocator(int8):
     nonlocal lens
     hp.fill_new_pages(lens)
     hc.page_token_indices = torch.from_numpy(hp.get_page_token_indices(lens)).to(DEV)
-    out = kern(xq, xk, xv, None, hc)
+    out = kern_h(xq, xk, xv, None, hc)
     lens = np.where(lens == 0, 0, lens + 1).astype(np.int32)
     return out
+
+  def same_output(got, want, what):
+    if not fused:
+      assert torch.equal(got, want), what
+      return
+    live = torch.from_numpy(lens > 0).to(DEV)  # inactive slots: nothing is attended
+    err = (got.float() - want.float()).abs()[live]
+    assert torch.all(err <= 1e-2 + 1e-2 * want.float().abs()[live]), f"{what}: max err {err.max():.4g}"
 
   def new_inputs():
     for t in (xq, xk, xv):
@@ -244,7 +259,7 @@ def test_paged_decode_steps_device_allocator_equals_host_allocator(int8):
     new_inputs()
     want = host_step()
     device_step()
-    assert torch.equal(out_d, want), f"eager step {step}"
+    same_output(out_d, want, f"eager step {step}")
     compare(f"eager step {step}")
   graph = torch.cuda.CUDAGraph()
   snapshot = [t.clone() for t in (dp._mem, dlens, dc.cache_k, dc.cache_v)] + (
@@ -260,6 +275,6 @@ def test_paged_decode_steps_device_allocator_equals_host_allocator(int8):
     torch.cuda.synchronize()
     graph.replay()
     torch.cuda.synchronize()
-    assert torch.equal(out_d, want), f"replay {step}"
+    same_output(out_d, want, f"replay {step}")
     compare(f"replay {step}")
   dp.check()
