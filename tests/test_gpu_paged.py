@@ -152,3 +152,86 @@ def test_int8_pages_equal_quantise_then_row_write(hs, sdt):
     want_vs[:, page, tok % ps] = wvs[slot, :, 0, 0]
   assert torch.equal(ck.cpu(), want_k) and torch.equal(cv.cpu(), want_v)
   assert torch.equal(ks.cpu(), want_ks) and torch.equal(vs.cpu(), want_vs)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "int8_codes", "int8_raw", "int8_raw_perhead_bf16"])
+def test_paged_attention_appends_the_token_itself(kind):
+  """new_to_pages: the attention launch writes the step's token to position
+  lens[b] of its slot's pages and attends it.  Pages and scale pages must be
+  what the separate append launch writes, bit for bit - inactive slots (length
+  0) and a full slot untouched; outputs those of attention after that append
+  (attention tolerance: the token is summed first, not last)."""
+  from jetstream_pt_amd import attention_kernel as ak
+  from jetstream_pt_amd import cache_manager as cm
+  from jetstream_pt_amd.quantize import quantize_kv
+  from oracle import attention as OA
+  g = torch.Generator().manual_seed(77)
+  rng = np.random.default_rng(77)
+  hq, hkv, p, ps, d, mp = 16, 4, 96, 32, 128, 4
+  lens = np.array([0, 1, 31, 32, 64, 100, 127, 128, 5, 0, 96], dtype=np.int32)  # 128 = a full slot (4 pages)
+  b = len(lens)
+  perm = rng.permutation(p - 1).astype(np.int32)  # page p-1 is the sentinel
+  table = np.full((b, mp), p - 1, dtype=np.int32)
+  at = 0
+  for bi, n in enumerate(lens):
+    need = min(mp, n // ps + 1) if n else 0  # the page of position n is there already
+    table[bi, :need] = perm[at:at + need]
+    at += need
+  int8 = kind != "bf16"
+  per_head = kind.endswith("perhead_bf16")
+  sdt = torch.bfloat16 if per_head else torch.float32
+  hs = hkv if per_head else 1
+  if int8:
+    kp = torch.randint(-127, 128, (hkv, p, ps, d), generator=g, dtype=torch.int8)
+    vp = torch.randint(-127, 128, (hkv, p, ps, d), generator=g, dtype=torch.int8)
+    ksp = (torch.rand((hs, p, ps), generator=g) * 0.045 + 0.005).to(sdt)
+    vsp = (torch.rand((hs, p, ps), generator=g) * 0.045 + 0.005).to(sdt)
+  else:
+    kp = torch.randn((hkv, p, ps, d), generator=g).to(torch.bfloat16)
+    vp = torch.randn((hkv, p, ps, d), generator=g).to(torch.bfloat16)
+    ksp = vsp = None
+  q = torch.randn((b, hq, d), generator=g).to(torch.bfloat16)
+  xk = torch.randn((b, hkv, 1, d), generator=g).to(torch.bfloat16)
+  xv = torch.randn((b, hkv, 1, d), generator=g).to(torch.bfloat16)
+  dev = lambda t: None if t is None else t.to(DEV)
+  gq, gxk, gxv, glens, gtable = dev(q), dev(xk), dev(xv), torch.from_numpy(lens).to(DEV), torch.from_numpy(table).to(DEV)
+
+  # reference flow: the separate append launch on a copy, then attention over lens + 1
+  active = np.nonzero((lens > 0) & (lens < mp * ps))[0]
+  idx = np.stack([table[active, lens[active] // ps], np.arange(len(active)) * ps + lens[active] % ps, active]).astype(np.int32)
+  wk, wv, wks, wvs = dev(kp.clone()), dev(vp.clone()), dev(None if ksp is None else ksp.clone()), dev(None if vsp is None else vsp.clone())
+  if int8:
+    ref = cm.Int8PageKVCacheGenerate(wk, wv, wks, wvs, None, idx, env=genv(p, ps))
+  else:
+    ref = cm.PageKVCacheGenerate(wk, wv, None, idx, env=genv(p, ps))
+  ref.update(gxk, gxv, 0)
+  after = np.where((lens > 0) & (lens < mp * ps), lens + 1, lens).astype(np.int32)
+  want = OA.paged_attention(q.float(), wk.cpu(), wv.cpu(), torch.from_numpy(after), torch.from_numpy(table), sm_scale=1.0,
+                            k_scale_pages=None if wks is None else wks.cpu().float(),
+                            v_scale_pages=None if wvs is None else wvs.cpu().float())
+
+  fk, fv, fks, fvs = dev(kp.clone()), dev(vp.clone()), dev(None if ksp is None else ksp.clone()), dev(None if vsp is None else vsp.clone())
+  if kind == "bf16":
+    append = dict(new_key=gxk, new_value=gxv)
+  elif kind == "int8_codes":
+    ck, cv, cks, cvs = quantize_kv(gxk, gxv, rounding="trunc", scale_heads=hs, scale_dtype=sdt)
+    append = dict(new_key=ck, new_value=cv, new_k_scaler=cks, new_v_scaler=cvs)
+  else:
+    append = dict(new_key=torch.empty((b, hkv, 1, d), dtype=torch.int8, device=DEV),
+                  new_value=torch.empty((b, hkv, 1, d), dtype=torch.int8, device=DEV),
+                  new_k_scaler=torch.empty((b, hs), dtype=sdt, device=DEV),
+                  new_v_scaler=torch.empty((b, hs), dtype=sdt, device=DEV),
+                  new_key_raw=gxk, new_value_raw=gxv, new_rounding="trunc")
+  got = ak.call_paged_attention(None, gq, fk, fv, glens, gtable, sm_scale=1.0, k_scaler=fks, v_scaler=fvs, append=append)
+  assert torch.equal(fk, wk) and torch.equal(fv, wv), "pages"
+  if int8:
+    assert torch.equal(fks, wks) and torch.equal(fvs, wvs), "scale pages"
+  live = torch.from_numpy((lens > 0) & (lens < mp * ps))
+  err = (got.float().cpu() - want.float()).abs()[live]
+  assert torch.all(err <= 1e-2 + 1e-2 * want.float().abs()[live]), f"max err {err.max():.4g}"
+  # a shape the streaming kernel does not take is refused, not half done
+  with pytest.raises(ValueError):
+    ak.call_paged_attention(None, gq[:, :, :64].contiguous(), fk[..., :64].contiguous(), fv[..., :64].contiguous(),
+                            glens, gtable, sm_scale=1.0, k_scaler=fks, v_scaler=fvs,
+                            append={k_: (v_[..., :64].contiguous() if torch.is_tensor(v_) and v_.dim() == 4 else v_)
+                                    for k_, v_ in append.items()})
