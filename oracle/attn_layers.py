@@ -10,7 +10,6 @@ The reference pads a single query row to two rows on some branches
 row never influences row 0, so it is not restated.
 """
 
-import torch
 
 from . import attention as A
 

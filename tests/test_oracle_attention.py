@@ -4,7 +4,6 @@ reference holds."""
 
 import math
 
-import numpy as np
 import pytest
 import torch
 

@@ -1,7 +1,6 @@
 """Pins the oracle's restatement of the engine's prefill -> decode insert
 (engine.py:371-626) by brute force on small shapes and by hand-worked cases."""
 
-import numpy as np
 import torch
 
 from oracle import Env
