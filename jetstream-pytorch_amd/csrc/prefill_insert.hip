@@ -148,14 +148,17 @@ __global__ void __launch_bounds__(256) prefill_insert_kernel(InsertParams p) {
   if (threadIdx.x < groups) store_from_f32(scale_out, scale_index(threadIdx.x), a.scale_dtype, s_scale[threadIdx.x]);
 }
 
-// The common quantising shape - bf16 prompt, heads * dim == 1024 - four tokens
-// a workgroup: a thread keeps its four elements of each token in registers
-// between the absmax pass and the quantise pass, so the prompt is read once
-// and four times as many bytes are in flight per workgroup.  Same op order.
-constexpr int kTokensPerBlock = 4;
+// The common quantising shape - bf16 prompt, heads * dim == 1024 - eight tokens
+// a workgroup, two at a time: 128 threads a token, each keeping its eight
+// elements (one 16-byte load) of four tokens in registers between the absmax
+// pass and the quantise pass, so the prompt is read once, in wide loads that
+// are all issued before the first wait.  Same op order as the general kernel.
+constexpr int kTokensPerBlock = 8;
 template <bool BF16_MATH>
 __global__ void __launch_bounds__(256) prefill_insert_quant4_kernel(InsertParams p) {
   const jpt_prefill_insert_args& a = p.a;
+  constexpr int kPasses = kTokensPerBlock / 2;
+  const int half = threadIdx.x >> 7;  // which of the pass's two tokens
   const int t0 = blockIdx.x * kTokensPerBlock;
   const bool is_v = blockIdx.y == 1;
   const int layer = blockIdx.z;
@@ -166,28 +169,30 @@ __global__ void __launch_bounds__(256) prefill_insert_quant4_kernel(InsertParams
   const uint16_t* src = static_cast<const uint16_t*>(is_v ? a.src_v : a.src_k) + layer * a.src_layer_stride;
   char* dst = static_cast<char*>(is_v ? a.dst_v : a.dst_k) + layer * a.dst_layer_stride;
   void* scale_out = static_cast<char*>(is_v ? a.v_scale : a.k_scale) + layer * a.scale_layer_stride * esz_scale;
-  const int i0 = 4 * threadIdx.x, h = i0 / D, d = i0 - h * D;
+  const int i0 = 8 * (threadIdx.x & 127), h = i0 / D, d = i0 - h * D;
   const int groups = a.scale_heads;
   const int64_t head_stride = a.src_head_stride > 0 ? a.src_head_stride : static_cast<int64_t>(a.tokens) * D;
 
-  // All four tokens' loads are issued before anything waits for one of them
-  // (addresses clamped into the prompt, results masked afterwards), and the
-  // page ids likewise: one memory round trip a workgroup, not one a token.
-  uint2 raw[kTokensPerBlock];
+  // every load of the workgroup before anything waits for one (addresses
+  // clamped into the prompt, results masked afterwards); page ids likewise
+  uint4 raw[kPasses];
 #pragma unroll
-  for (int j = 0; j < kTokensPerBlock; ++j) {
-    const int t = min(t0 + j, a.tokens - 1);
-    raw[j] = *reinterpret_cast<const uint2*>(src + h * head_stride + static_cast<int64_t>(t) * D + d);
+  for (int j = 0; j < kPasses; ++j) {
+    const int t = min(t0 + 2 * j + half, a.tokens - 1);
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 w = __builtin_nontemporal_load(
+        reinterpret_cast<const u32x4*>(src + h * head_stride + static_cast<int64_t>(t) * D + d));  // read once
+    raw[j] = make_uint4(w.x, w.y, w.z, w.w);
   }
-  int page_of[kTokensPerBlock];
+  int page_of[kPasses];
 #pragma unroll
-  for (int j = 0; j < kTokensPerBlock; ++j)
-    page_of[j] = paged ? a.page_ids[min(t0 + j, rows - 1) / a.page_size] : 0;
-  float x[kTokensPerBlock][4], m[kTokensPerBlock];
-  int64_t pool_row[kTokensPerBlock];  // dense: position in the slot's row; paged: row in the pool; -1: nothing to write
+  for (int j = 0; j < kPasses; ++j)
+    page_of[j] = paged ? a.page_ids[min(t0 + 2 * j + half, rows - 1) / a.page_size] : 0;
+  float x[kPasses][8], m[kPasses];
+  int64_t pool_row[kPasses];  // dense: position in the slot's row; paged: row in the pool; -1: nothing to write
 #pragma unroll
-  for (int j = 0; j < kTokensPerBlock; ++j) {
-    const int t = t0 + j;
+  for (int j = 0; j < kPasses; ++j) {
+    const int t = t0 + 2 * j + half;
     pool_row[j] = -1;
     if (t < rows) {
       if (paged) {
@@ -199,60 +204,65 @@ __global__ void __launch_bounds__(256) prefill_insert_quant4_kernel(InsertParams
       }
     }
     const bool live = t < a.tokens;
-    x[j][0] = live ? __uint_as_float(raw[j].x << 16) : 0.f;
-    x[j][1] = live ? __uint_as_float(raw[j].x & 0xffff0000u) : 0.f;
-    x[j][2] = live ? __uint_as_float(raw[j].y << 16) : 0.f;
-    x[j][3] = live ? __uint_as_float(raw[j].y & 0xffff0000u) : 0.f;
-    m[j] = fmaxf(fmaxf(fabsf(x[j][0]), fabsf(x[j][1])), fmaxf(fabsf(x[j][2]), fabsf(x[j][3])));
+    const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+    m[j] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[j][2 * i] = live ? __uint_as_float(w[i] << 16) : 0.f;
+      x[j][2 * i + 1] = live ? __uint_as_float(w[i] & 0xffff0000u) : 0.f;
+      m[j] = fmaxf(m[j], fmaxf(fabsf(x[j][2 * i]), fabsf(x[j][2 * i + 1])));
+    }
   }
-  __shared__ float s_red[kTokensPerBlock][4];
+  __shared__ float s_red[kPasses][4];
   if (groups == 1) {
 #pragma unroll
-    for (int j = 0; j < kTokensPerBlock; ++j) {
+    for (int j = 0; j < kPasses; ++j) {
       for (int off = 32; off > 0; off >>= 1) m[j] = fmaxf(m[j], __shfl_xor(m[j], off));
       if ((threadIdx.x & 63) == 0) s_red[j][threadIdx.x >> 6] = m[j];
     }
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < kTokensPerBlock; ++j)
-      m[j] = fmaxf(fmaxf(s_red[j][0], s_red[j][1]), fmaxf(s_red[j][2], s_red[j][3]));
+    for (int j = 0; j < kPasses; ++j) m[j] = fmaxf(s_red[j][2 * half], s_red[j][2 * half + 1]);
   } else {
-    // a head's D / 4 threads are consecutive; D / 4 is a power of two <= 64
+    // a head's D / 8 threads are consecutive; D / 8 is a power of two <= 64
 #pragma unroll
-    for (int j = 0; j < kTokensPerBlock; ++j)
-      for (int off = D / 8; off > 0; off >>= 1) m[j] = fmaxf(m[j], __shfl_xor(m[j], off));
+    for (int j = 0; j < kPasses; ++j)
+      for (int off = D / 16; off > 0; off >>= 1) m[j] = fmaxf(m[j], __shfl_xor(m[j], off));
   }
 #pragma unroll
-  for (int j = 0; j < kTokensPerBlock; ++j) {
+  for (int j = 0; j < kPasses; ++j) {
     if (pool_row[j] < 0) continue;
     const int64_t row = paged ? static_cast<int64_t>(h) * a.total_pages * a.page_size + pool_row[j]
                               : (static_cast<int64_t>(a.slot) * H + h) * a.seq + pool_row[j];
-    uint32_t* out = reinterpret_cast<uint32_t*>(dst + row * D + d);
-    if (t0 + j >= a.tokens) {  // paged only: the tail of the last page is zero-filled
-      *out = 0u;
+    uint2* out = reinterpret_cast<uint2*>(dst + row * D + d);
+    if (t0 + 2 * j + half >= a.tokens) {  // paged only: the tail of the last page is zero-filled
+      *out = make_uint2(0u, 0u);
       continue;
     }
     float amax = m[j];
     if (a.rounding == JPT_ROUND_RNE) amax = fmaxf(amax, rnd<BF16_MATH>(1e-5f));
     const float s = rnd<BF16_MATH>(amax / 127.0f);
-    int code[4];
+    uint32_t code[8];
     if (a.rounding == JPT_ROUND_TRUNC) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < 8; ++i) {
         const float q = rnd<BF16_MATH>(x[j][i] / s);
-        code[i] = (q != q) ? 0 : static_cast<int>(q);
+        code[i] = static_cast<uint32_t>((q != q) ? 0 : static_cast<int>(q)) & 0xffu;
       }
     } else {
       const float r = rnd<BF16_MATH>(1.0f / s);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < 8; ++i) {
         const float q = rnd<BF16_MATH>(x[j][i] * r);
-        code[i] = static_cast<int>(fminf(fmaxf(rintf(q), -128.f), 127.f));
+        code[i] = static_cast<uint32_t>(static_cast<int>(fminf(fmaxf(rintf(q), -128.f), 127.f))) & 0xffu;
       }
     }
-    *out = (static_cast<uint32_t>(code[0]) & 0xffu) | ((static_cast<uint32_t>(code[1]) & 0xffu) << 8) |
-           ((static_cast<uint32_t>(code[2]) & 0xffu) << 16) | (static_cast<uint32_t>(code[3]) << 24);
-    if (groups == 1 ? threadIdx.x == 0 : d == 0) {
+    // written once, read by later launches only: keep it out of the way of the prompt being read
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 packed = {code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24),
+                          code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24)};
+    __builtin_nontemporal_store(packed, reinterpret_cast<u32x2*>(out));
+    if (groups == 1 ? (threadIdx.x & 127) == 0 : d == 0) {
       const int g = groups == 1 ? 0 : h;
       const int64_t idx = paged ? static_cast<int64_t>(g) * a.total_pages * a.page_size + pool_row[j]
                                 : (static_cast<int64_t>(a.slot) * groups + g) * a.seq + pool_row[j];
@@ -302,10 +312,12 @@ extern "C" int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void*
   InsertParams p{*args};
   if (p.a.n_layers <= 0) p.a.n_layers = 1;
   JPT_REQUIRE(p.a.n_layers <= 65535, "n_layers out of range");
-  const int d4 = a.dim / 4;
-  const bool four = quant && a.tokens > 0 && a.in_dtype == JPT_BF16 && a.heads * a.dim == 1024 &&
-                    (a.scale_heads == 1 || (d4 <= 64 && (d4 & (d4 - 1)) == 0)) && aligned(a.src_k, 8) &&
-                    aligned(a.src_v, 8) && (a.src_head_stride == 0 || a.src_head_stride % 4 == 0);
+  const int d8 = a.dim / 8;  // threads a head in the wide kernel
+  const bool four = quant && a.tokens > 0 && a.in_dtype == JPT_BF16 && a.heads * a.dim == 1024 && a.dim % 8 == 0 &&
+                    (a.scale_heads == 1 || (d8 <= 64 && (d8 & (d8 - 1)) == 0)) && aligned(a.src_k, 16) &&
+                    aligned(a.src_v, 16) && (a.src_head_stride == 0 || a.src_head_stride % 8 == 0) &&
+                    a.src_layer_stride % 8 == 0 && aligned(a.dst_k, 8) && aligned(a.dst_v, 8) &&
+                    a.dst_layer_stride % 8 == 0;
   if (four) {
     dim3 grid4((rows + kTokensPerBlock - 1) / kTokensPerBlock, 2, p.a.n_layers);
     if (a.scale_dtype == JPT_BF16)
