@@ -49,7 +49,7 @@ PROBE_COPY_BYTES = 1 << 30
 # headline workload, from hardware counters (FETCH_SIZE + WRITE_SIZE, each
 # calibrated on a 1 GiB copy; see --probe-traffic).  A recorded measurement,
 # not computed here.
-MEASURED_ATTN_TRAFFIC_BYTES = 157_490_000
+MEASURED_ATTN_TRAFFIC_BYTES = 157_450_000
 DEV = "cuda:0"
 
 
