@@ -228,6 +228,25 @@ typedef struct {
 
 int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void* stream);
 
+/* The same insert for layers that are tensors of their own (the reference's
+ * unstacked DecodeState: a list of per-layer caches, engine.py:371-488 loops
+ * over them inside one jitted program): one launch for up to 64 layers, the
+ * pointers travelling in the kernel arguments.  `args` gives everything but
+ * the six tensor pointers and the layer strides, which are ignored; `layers`
+ * is a HOST array of n_layers entries (k_scale/v_scale NULL for a copy). */
+typedef struct {
+  const void* src_k;
+  const void* src_v;
+  void* dst_k;
+  void* dst_v;
+  void* k_scale;
+  void* v_scale;
+} jpt_insert_layer;
+
+int32_t jpt_prefill_insert_layers(const jpt_prefill_insert_args* args,
+                                  const jpt_insert_layer* layers,
+                                  int32_t n_layers, void* stream);
+
 /* ------------------------------------------------------------------------
  * Decode attention.
  *

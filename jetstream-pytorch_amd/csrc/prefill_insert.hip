@@ -9,9 +9,36 @@
 namespace jpt {
 namespace {
 
+// Layers that are tensors of their own (no common stride) come as a table of
+// pointers inside the kernel arguments.
+constexpr int kTableLayers = 64;
 struct InsertParams {
   jpt_prefill_insert_args a;
+  int32_t use_table;
+  const void* src_k[kTableLayers];
+  const void* src_v[kTableLayers];
+  void* dst_k[kTableLayers];
+  void* dst_v[kTableLayers];
+  void* k_scale[kTableLayers];
+  void* v_scale[kTableLayers];
 };
+
+// Source, destination and scale tensor of (layer, K|V): the table's, or the
+// first layer's moved on by the layer strides.
+__device__ __forceinline__ void layer_tensors(const InsertParams& p, int layer, bool is_v, int esz_in, int esz_out,
+                                              int esz_scale, const void** src, char** dst, void** scale) {
+  const jpt_prefill_insert_args& a = p.a;
+  if (p.use_table) {
+    *src = is_v ? p.src_v[layer] : p.src_k[layer];
+    *dst = static_cast<char*>(is_v ? p.dst_v[layer] : p.dst_k[layer]);
+    *scale = is_v ? p.v_scale[layer] : p.k_scale[layer];
+    return;
+  }
+  *src = static_cast<const char*>(is_v ? a.src_v : a.src_k) + layer * a.src_layer_stride * esz_in;
+  *dst = static_cast<char*>(is_v ? a.dst_v : a.dst_k) + layer * a.dst_layer_stride * esz_out;
+  void* s0 = is_v ? a.v_scale : a.k_scale;
+  *scale = s0 == nullptr ? nullptr : static_cast<char*>(s0) + layer * a.scale_layer_stride * esz_scale;
+}
 
 template <bool ROUND_BF16>
 __device__ __forceinline__ float rnd(float x) {
@@ -49,10 +76,10 @@ __global__ void __launch_bounds__(256) prefill_insert_kernel(InsertParams p) {
   const int esz_in = a.in_dtype == JPT_F32 ? 4 : a.in_dtype == JPT_BF16 ? 2 : 1;
   const int esz_out = quant ? 1 : esz_in;
   const int esz_scale = a.scale_dtype == JPT_F32 ? 4 : 2;
-  const void* src = static_cast<const char*>(is_v ? a.src_v : a.src_k) + layer * a.src_layer_stride * esz_in;
-  char* dst = static_cast<char*>(is_v ? a.dst_v : a.dst_k) + layer * a.dst_layer_stride * esz_out;
-  void* scale_out = (is_v ? a.v_scale : a.k_scale) == nullptr ? nullptr
-      : static_cast<char*>(is_v ? a.v_scale : a.k_scale) + layer * a.scale_layer_stride * esz_scale;
+  const void* src;
+  char* dst;
+  void* scale_out;
+  layer_tensors(p, layer, is_v, esz_in, esz_out, esz_scale, &src, &dst, &scale_out);
 
   // destination row of (this token, head h): element index row * D
   int64_t pool_row = 0;  // dense: position in the slot's row; paged: row in the pool
@@ -166,9 +193,11 @@ __global__ void __launch_bounds__(256) prefill_insert_quant4_kernel(InsertParams
   const int H = a.heads, D = a.dim;
   const int rows = paged ? a.n_pages * a.page_size : a.tokens;
   const int esz_scale = a.scale_dtype == JPT_F32 ? 4 : 2;
-  const uint16_t* src = static_cast<const uint16_t*>(is_v ? a.src_v : a.src_k) + layer * a.src_layer_stride;
-  char* dst = static_cast<char*>(is_v ? a.dst_v : a.dst_k) + layer * a.dst_layer_stride;
-  void* scale_out = static_cast<char*>(is_v ? a.v_scale : a.k_scale) + layer * a.scale_layer_stride * esz_scale;
+  const void* src_any;
+  char* dst;
+  void* scale_out;
+  layer_tensors(p, layer, is_v, 2, 1, esz_scale, &src_any, &dst, &scale_out);
+  const uint16_t* src = static_cast<const uint16_t*>(src_any);
   const int i0 = 8 * (threadIdx.x & 127), h = i0 / D, d = i0 - h * D;
   const int groups = a.scale_heads;
   const int64_t head_stride = a.src_head_stride > 0 ? a.src_head_stride : static_cast<int64_t>(a.tokens) * D;
@@ -274,30 +303,58 @@ __global__ void __launch_bounds__(256) prefill_insert_quant4_kernel(InsertParams
 }  // namespace
 }  // namespace jpt
 
-extern "C" int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void* stream) {
-  using namespace jpt;
-  JPT_REQUIRE(args != nullptr, "args is NULL");
-  const jpt_prefill_insert_args& a = *args;
-  JPT_REQUIRE(a.src_k && a.src_v && a.dst_k && a.dst_v, "NULL tensor argument");
+namespace jpt {
+namespace {
+
+// Checks and launches.  layers == nullptr: the tensors of args, n_layers of them
+// a layer stride apart; else a table of at most kTableLayers layers.
+int32_t insert_launch(const jpt_prefill_insert_args& a, const jpt_insert_layer* layers, int32_t n_table, void* stream) {
   JPT_REQUIRE(a.tokens >= 0 && a.heads > 0 && a.dim > 0, "tokens, heads, dim out of range");
   JPT_REQUIRE(a.dim % 4 == 0, "dim must be a multiple of 4");
   JPT_REQUIRE(a.in_dtype == JPT_BF16 || a.in_dtype == JPT_F32 || a.in_dtype == JPT_I8, "bad in_dtype");
   const bool quant = a.dst_dtype == JPT_I8 && a.in_dtype != JPT_I8;
   JPT_REQUIRE(quant || a.dst_dtype == a.in_dtype, "dst_dtype must be in_dtype (copy) or int8 (quantise)");
   const int esz = a.in_dtype == JPT_F32 ? 4 : a.in_dtype == JPT_BF16 ? 2 : 1;
-  JPT_REQUIRE(aligned(a.src_k, 4 * esz) && aligned(a.src_v, 4 * esz), "source rows must be aligned to four elements");
+  const int esz_out = quant ? 1 : esz;
   JPT_REQUIRE(a.src_head_stride == 0 || (a.src_head_stride >= static_cast<int64_t>(a.tokens) * a.dim && a.src_head_stride % 4 == 0),
               "src_head_stride must cover the tokens and be a multiple of 4");
-  JPT_REQUIRE(a.src_layer_stride % 4 == 0 && a.dst_layer_stride % 4 == 0, "layer strides must be multiples of 4");
-  const int esz_out = quant ? 1 : esz;
-  JPT_REQUIRE(aligned(a.dst_k, 4 * esz_out) && aligned(a.dst_v, 4 * esz_out), "destination must be aligned to four elements");
   if (quant) {
-    JPT_REQUIRE(a.k_scale && a.v_scale, "k_scale/v_scale are NULL");
     JPT_REQUIRE(a.scale_dtype == a.in_dtype || a.scale_dtype == JPT_F32, "scale_dtype must equal in_dtype or be f32");
     JPT_REQUIRE(a.scale_heads == 1 || a.scale_heads == a.heads, "scale_heads must be 1 or heads");
     JPT_REQUIRE(a.scale_heads <= 64, "per-head scales support at most 64 heads");
-    JPT_REQUIRE(a.scale_heads == 1 || a.dim % 4 == 0, "dim must be a multiple of 4");
     JPT_REQUIRE(a.rounding == JPT_ROUND_TRUNC || a.rounding == JPT_ROUND_RNE, "bad rounding mode");
+  }
+  InsertParams p{};
+  p.a = a;
+  bool wide_ok = true;  // every tensor is aligned for the wide quantising kernel
+  auto check_layer = [&](const void* sk, const void* sv, const void* dk, const void* dv, const void* ks,
+                         const void* vs) -> int32_t {
+    JPT_REQUIRE(sk && sv && dk && dv, "NULL tensor argument");
+    JPT_REQUIRE(aligned(sk, 4 * esz) && aligned(sv, 4 * esz), "source rows must be aligned to four elements");
+    JPT_REQUIRE(aligned(dk, 4 * esz_out) && aligned(dv, 4 * esz_out), "destination must be aligned to four elements");
+    if (quant) JPT_REQUIRE(ks && vs, "k_scale/v_scale are NULL");
+    wide_ok = wide_ok && aligned(sk, 16) && aligned(sv, 16) && aligned(dk, 8) && aligned(dv, 8);
+    return JPT_OK;
+  };
+  if (layers) {
+    JPT_REQUIRE(n_table >= 1 && n_table <= kTableLayers, "1..%d layers a table", kTableLayers);
+    p.use_table = 1;
+    p.a.n_layers = n_table;
+    for (int l = 0; l < n_table; ++l) {
+      const jpt_insert_layer& t = layers[l];
+      const int32_t st = check_layer(t.src_k, t.src_v, t.dst_k, t.dst_v, t.k_scale, t.v_scale);
+      if (st != JPT_OK) return st;
+      p.src_k[l] = t.src_k; p.src_v[l] = t.src_v;
+      p.dst_k[l] = t.dst_k; p.dst_v[l] = t.dst_v;
+      p.k_scale[l] = t.k_scale; p.v_scale[l] = t.v_scale;
+    }
+  } else {
+    const int32_t st = check_layer(a.src_k, a.src_v, a.dst_k, a.dst_v, a.k_scale, a.v_scale);
+    if (st != JPT_OK) return st;
+    JPT_REQUIRE(a.src_layer_stride % 4 == 0 && a.dst_layer_stride % 4 == 0, "layer strides must be multiples of 4");
+    if (p.a.n_layers <= 0) p.a.n_layers = 1;
+    JPT_REQUIRE(p.a.n_layers <= 65535, "n_layers out of range");
+    wide_ok = wide_ok && a.src_layer_stride % 8 == 0 && a.dst_layer_stride % 8 == 0;
   }
   int32_t rows = a.tokens;
   if (a.page_ids) {
@@ -309,15 +366,10 @@ extern "C" int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void*
     JPT_REQUIRE(a.tokens <= a.seq, "%d tokens do not fit a cache of %d positions", a.tokens, a.seq);
   }
   if (rows == 0) return JPT_OK;
-  InsertParams p{*args};
-  if (p.a.n_layers <= 0) p.a.n_layers = 1;
-  JPT_REQUIRE(p.a.n_layers <= 65535, "n_layers out of range");
   const int d8 = a.dim / 8;  // threads a head in the wide kernel
-  const bool four = quant && a.tokens > 0 && a.in_dtype == JPT_BF16 && a.heads * a.dim == 1024 && a.dim % 8 == 0 &&
-                    (a.scale_heads == 1 || (d8 <= 64 && (d8 & (d8 - 1)) == 0)) && aligned(a.src_k, 16) &&
-                    aligned(a.src_v, 16) && (a.src_head_stride == 0 || a.src_head_stride % 8 == 0) &&
-                    a.src_layer_stride % 8 == 0 && aligned(a.dst_k, 8) && aligned(a.dst_v, 8) &&
-                    a.dst_layer_stride % 8 == 0;
+  const bool four = quant && wide_ok && a.tokens > 0 && a.in_dtype == JPT_BF16 && a.heads * a.dim == 1024 &&
+                    a.dim % 8 == 0 && (a.scale_heads == 1 || (d8 <= 64 && (d8 & (d8 - 1)) == 0)) &&
+                    (a.src_head_stride == 0 || a.src_head_stride % 8 == 0);
   if (four) {
     dim3 grid4((rows + kTokensPerBlock - 1) / kTokensPerBlock, 2, p.a.n_layers);
     if (a.scale_dtype == JPT_BF16)
@@ -333,3 +385,29 @@ extern "C" int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void*
     hipLaunchKernelGGL(prefill_insert_kernel<false>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), p);
   return launch_status("prefill_insert_kernel");
 }
+
+}  // namespace
+}  // namespace jpt
+
+extern "C" {
+
+int32_t jpt_prefill_insert(const jpt_prefill_insert_args* args, void* stream) {
+  using namespace jpt;
+  JPT_REQUIRE(args != nullptr, "args is NULL");
+  return insert_launch(*args, nullptr, 0, stream);
+}
+
+int32_t jpt_prefill_insert_layers(const jpt_prefill_insert_args* args, const jpt_insert_layer* layers,
+                                  int32_t n_layers, void* stream) {
+  using namespace jpt;
+  JPT_REQUIRE(args != nullptr && layers != nullptr, "NULL argument");
+  JPT_REQUIRE(n_layers >= 1, "n_layers must be positive");
+  for (int32_t l0 = 0; l0 < n_layers; l0 += kTableLayers) {
+    const int32_t n = n_layers - l0 < kTableLayers ? n_layers - l0 : kTableLayers;
+    const int32_t st = insert_launch(*args, layers + l0, n, stream);
+    if (st != JPT_OK) return st;
+  }
+  return JPT_OK;
+}
+
+}  // extern "C"

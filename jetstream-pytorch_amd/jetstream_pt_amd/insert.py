@@ -4,7 +4,8 @@ Mirrors the cache and bookkeeping part of the reference engine's insert
 (jetstream_pt/engine.py): `_insert_no_wrap` (:371-488), `_insert_wrap`
 (:491-581), `insert` (:606-626) and, for int8 pages, the paged insert
 (:583-604 with page_attention_manager.py:83-142).  Caches are updated in
-place by one kernel launch per layer (K and V together); with a quantised
+place by one kernel launch for all layers (K and V together; per-layer
+tensors travel as a pointer table); with a quantised
 cache the prompt is quantised per token over (heads, dim) by the reference's
 insert quantiser (quantize.py:58-75: round half to even, clamp, eps 1e-5) in
 the prompt's dtype.
@@ -41,6 +42,7 @@ def insert_prefix_caches(prefix_caches, caches, cache_scales, slot, start, *, ro
   float caches take a copy (cast to the cache dtype first).
   """
   n_layers = len(prefix_caches)
+  layers, keep, common, shape = [], [], None, None
   for layer, (newk, newv) in enumerate(prefix_caches):
     k, v = _layer_views(caches, layer, n_layers)
     k, v = _ffi.dev(k, "cache_k"), _ffi.dev(v, "cache_v")
@@ -54,18 +56,32 @@ def insert_prefix_caches(prefix_caches, caches, cache_scales, slot, start, *, ro
     newk, newv = _ffi.dev(newk.contiguous(), "prefix key"), _ffi.dev(newv.contiguous(), "prefix value")
     if newk.shape != (heads, tokens, dim):
       raise ValueError(f"prefix key {tuple(newk.shape)} does not match cache {tuple(k.shape)}")
-    a = _ffi.PrefillInsertArgs(
-        src_k=_ffi.ptr(newk), src_v=_ffi.ptr(newv), dst_k=_ffi.ptr(k), dst_v=_ffi.ptr(v),
-        tokens=tokens, heads=heads, dim=dim, slot=int(slot), batch=batch, seq=seq,
-        start=int(start), in_dtype=_ffi.dtype_code(newk.dtype),
-        dst_dtype=_ffi.dtype_code(k.dtype))
+    ks = vs = None
     if quant:
       ks, vs = _layer_views(cache_scales, layer, n_layers)
       ks, vs = _ffi.dev(ks, "k_scaler"), _ffi.dev(vs, "v_scaler")
-      a.k_scale, a.v_scale = _ffi.ptr(ks), _ffi.ptr(vs)
-      a.scale_dtype, a.scale_heads = _ffi.dtype_code(ks.dtype), ks.shape[1]
-      a.rounding = _rounding_code(rounding)
-    _ffi.check(_ffi.lib.jpt_prefill_insert(a, _ffi.stream()))
+    this = (tuple(k.shape), k.dtype, tuple(newk.shape), newk.dtype, None if ks is None else (ks.dtype, tuple(ks.shape)))
+    if shape is not None and this != shape:
+      raise ValueError("the layers of one insert must agree in shape and dtype")
+    shape = this
+    if common is None:
+      common = _ffi.PrefillInsertArgs(
+          tokens=tokens, heads=heads, dim=dim, slot=int(slot), batch=batch, seq=seq,
+          start=int(start), in_dtype=_ffi.dtype_code(newk.dtype), dst_dtype=_ffi.dtype_code(k.dtype))
+      if quant:
+        common.scale_dtype, common.scale_heads = _ffi.dtype_code(ks.dtype), ks.shape[1]
+        common.rounding = _rounding_code(rounding)
+    layers.append((_ffi.ptr(newk), _ffi.ptr(newv), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(ks), _ffi.ptr(vs)))
+    keep += [newk, newv]
+  if layers:
+    _launch_layers(common, layers, keep)
+
+
+def _launch_layers(common, layers, keep):
+  """One launch for all the layers of `layers` (lists of six pointers)."""
+  table = (_ffi.InsertLayer * len(layers))(*[_ffi.InsertLayer(*l) for l in layers])
+  _ffi.check(_ffi.lib.jpt_prefill_insert_layers(common, table, len(layers), _ffi.stream()))
+  del keep
 
 
 def insert_prefix_pages_int8(prefix_caches, decode_caches, scale_pages, page_ids, *, rounding="rne"):
@@ -74,19 +90,56 @@ def insert_prefix_pages_int8(prefix_caches, decode_caches, scale_pages, page_ids
   page is zero-filled (as insert_prefill_cache does for float pages).
   decode_caches / scale_pages: per-layer lists of (k, v) pairs."""
   ids = _ffi.as_i32(page_ids, decode_caches[0][0].device)
+  layers, keep, common, shape = [], [ids], None, None
   for (newk, newv), (pk, pv), (ks, vs) in zip(prefix_caches, decode_caches, scale_pages):
     pk, pv = _ffi.dev(pk, "pages_k"), _ffi.dev(pv, "pages_v")
+    ks, vs = _ffi.dev(ks, "k_scale_pages"), _ffi.dev(vs, "v_scale_pages")
     heads, total, ps, dim = pk.shape
     if newk.dim() == 4:
       newk, newv = newk[0], newv[0]
     newk, newv = _ffi.dev(newk.contiguous(), "prefix key"), _ffi.dev(newv.contiguous(), "prefix value")
-    a = _ffi.PrefillInsertArgs(
-        src_k=_ffi.ptr(newk), src_v=_ffi.ptr(newv), dst_k=_ffi.ptr(pk), dst_v=_ffi.ptr(pv),
-        k_scale=_ffi.ptr(_ffi.dev(ks, "k_scale_pages")), v_scale=_ffi.ptr(_ffi.dev(vs, "v_scale_pages")),
-        page_ids=_ffi.ptr(ids), n_pages=ids.numel(), tokens=newk.shape[1], heads=heads, dim=dim,
-        total_pages=total, page_size=ps, in_dtype=_ffi.dtype_code(newk.dtype), dst_dtype=_ffi.I8,
-        scale_dtype=_ffi.dtype_code(ks.dtype), scale_heads=ks.shape[0], rounding=_rounding_code(rounding))
-    _ffi.check(_ffi.lib.jpt_prefill_insert(a, _ffi.stream()))
+    this = (tuple(pk.shape), tuple(newk.shape), newk.dtype, ks.dtype, tuple(ks.shape))
+    if shape is not None and this != shape:
+      raise ValueError("the layers of one insert must agree in shape and dtype")
+    shape = this
+    if common is None:
+      common = _ffi.PrefillInsertArgs(
+          page_ids=_ffi.ptr(ids), n_pages=ids.numel(), tokens=newk.shape[1], heads=heads, dim=dim,
+          total_pages=total, page_size=ps, in_dtype=_ffi.dtype_code(newk.dtype), dst_dtype=_ffi.I8,
+          scale_dtype=_ffi.dtype_code(ks.dtype), scale_heads=ks.shape[0], rounding=_rounding_code(rounding))
+    layers.append((_ffi.ptr(newk), _ffi.ptr(newv), _ffi.ptr(pk), _ffi.ptr(pv), _ffi.ptr(ks), _ffi.ptr(vs)))
+    keep += [newk, newv]
+  if layers:
+    _launch_layers(common, layers, keep)
+
+
+def insert_prefix_pages_copy(prefix_caches, decode_caches, page_ids):
+  """Float pages, all layers in one launch: token t of every layer's prompt
+  (1, heads, T, D) goes to page page_ids[t // ps], row t % ps, the rest of the
+  last page is zero-filled (insert_prefill_cache, page_attention_manager.py:
+  83-142).  Needs head_dim % 4 == 0 and layers of one shape and dtype; returns
+  False, having done nothing, when that does not hold."""
+  ids = _ffi.as_i32(page_ids, decode_caches[0][0].device)
+  layers, keep, common, shape = [], [ids], None, None
+  for (newk, newv), (pk, pv) in zip(prefix_caches, decode_caches):
+    if not (pk.is_cuda and pk.is_contiguous() and pv.is_contiguous()) or pk.dtype not in (torch.bfloat16, torch.float32):
+      return False
+    heads, total, ps, dim = pk.shape
+    newk, newv = newk.to(pk.dtype).contiguous(), newv.to(pv.dtype).contiguous()
+    this = (tuple(pk.shape), pk.dtype, tuple(newk.shape))
+    if dim % 4 != 0 or newk.dim() != 4 or newk.shape[0] != 1 or newk.shape[1] != heads or newk.shape[3] != dim \
+        or (shape is not None and this != shape) or not newk.is_cuda:
+      return False
+    shape = this
+    if common is None:
+      common = _ffi.PrefillInsertArgs(
+          page_ids=_ffi.ptr(ids), n_pages=ids.numel(), tokens=newk.shape[2], heads=heads, dim=dim,
+          total_pages=total, page_size=ps, in_dtype=_ffi.dtype_code(pk.dtype), dst_dtype=_ffi.dtype_code(pk.dtype))
+    layers.append((_ffi.ptr(newk), _ffi.ptr(newv), _ffi.ptr(pk), _ffi.ptr(pv), None, None))
+    keep += [newk, newv]
+  if layers:
+    _launch_layers(common, layers, keep)
+  return True
 
 
 def insert_prefix_pages_int8_stacked(prefix_k, prefix_v, pages_k, pages_v, k_scale_pages, v_scale_pages,

@@ -142,6 +142,10 @@ class PageAttentionManager:
       return decode_caches
     device = decode_caches[0][0].device
     ids = _ffi.as_i32(update_indexes, device)
+    if len(decode_caches) > 1:  # all layers in one launch where their shapes allow
+      from . import insert as _insert
+      if _insert.insert_prefix_pages_copy(prefill_caches, decode_caches, ids):
+        return decode_caches
     for (k, v), (pk, pv) in zip(prefill_caches, decode_caches):
       _ffi.dev(pk, "decode cache"), _ffi.dev(pv, "decode cache")
       heads, total, ps, dim = pk.shape
