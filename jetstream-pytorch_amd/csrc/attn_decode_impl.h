@@ -55,7 +55,8 @@ typedef __attribute__((address_space(3))) void* lds_ptr;
 #ifndef JPT_ATTN_EXPERIMENT_CUT
 // Development builds for timing experiments only (results are wrong): 1, 2 stop a
 // tile's work early; 3 skips an item's fold and output; 4 only the fold by the
-// last consumer to arrive; 5 the conversion of the query operand.
+// last consumer to arrive; 5 the conversion of the query operand; 6 the fold's
+// global stores.
 #define JPT_ATTN_EXPERIMENT_CUT 0
 #endif
 #ifndef JPT_ATTN_CONSUMERS
@@ -1061,6 +1062,10 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         o[0] += x.x * f; o[1] += x.y * f; o[2] += x.z * f; o[3] += x.w * f;
         o[4] += y.x * f; o[5] += y.y * f; o[6] += y.z * f; o[7] += y.w * f;
       }
+#if JPT_ATTN_EXPERIMENT_CUT == 6
+      asm volatile("" ::"v"(o[0] + o[1] + o[2] + o[3] + o[4] + o[5] + o[6] + o[7] + l + M));
+      continue;
+#endif
       if (it.n_chunks == 1) {
         const float inv = l > 0.f ? 1.f / l : 0.f;
         const uint4 packed = make_uint4(pack_bf16(o[0] * inv, o[1] * inv), pack_bf16(o[2] * inv, o[3] * inv),
