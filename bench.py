@@ -395,7 +395,7 @@ def run_gpu(args):
   def timed(fn, steps, warmup, before=None):
     """fn(i) enqueues step i.  Whole passes over the layers are replayed from
     one captured HIP graph where the workload allows (what a serving loop does
-    with a launch-bound decode step); a remainder of steps runs eagerly.
+    with a launch-bound decode step); a remainder of steps from a shorter one.
     before(), when given, is the eager per-pass work ahead of layer 0."""
     before = before or (lambda: None)
     warmup = (max(warmup, nl) + nl - 1) // nl * nl  # whole passes
@@ -404,15 +404,21 @@ def run_gpu(args):
         before()
       fn(i)
     torch.cuda.synchronize()
-    graph = None
-    if use_graph and steps >= nl:
-      graph = torch.cuda.CUDAGraph()
-      with torch.cuda.graph(graph):
-        for i in range(nl):
-          fn(i)
-      before()
-      graph.replay()
-      torch.cuda.synchronize()
+    graph = rest = None
+    if use_graph:
+      def capture(n):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+          for i in range(n):
+            fn(i)
+        before()
+        g.replay()
+        torch.cuda.synchronize()
+        return g
+      if steps >= nl:
+        graph = capture(nl)
+      if steps % nl:  # the steps left over after the whole passes: a shorter graph of their own
+        rest = capture(steps % nl)
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     done = 0
@@ -421,6 +427,10 @@ def run_gpu(args):
         before()
         graph.replay()
       done = steps // nl * nl
+    if rest is not None:
+      before()
+      rest.replay()
+      done = steps
     for i in range(done, steps):
       if i % nl == 0:
         before()
