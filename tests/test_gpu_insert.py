@@ -156,3 +156,28 @@ def test_int8_paged_insert_all_layers_in_one_launch():
     assert torch.equal(one[0][0][l], per[0][l][0]) and torch.equal(one[0][1][l], per[0][l][1])
     assert torch.equal(one[1][0][l], per[1][l][0]) and torch.equal(one[1][1][l], per[1][l][1])
   assert not torch.equal(one[0][0].cpu(), pk)
+
+
+@pytest.mark.parametrize("block", range(3))
+def test_random_dense_inserts(block):
+  """Randomly drawn insert shapes - stacked and per-layer caches, ring wrap,
+  copy and both quantiser kernels (heads * dim == 1024 takes the wide one),
+  one to five layers in one launch - bit for bit against the oracle."""
+  import numpy as np
+  for it in range(10):
+    seed = 500 + 100 * block + it
+    rng = np.random.default_rng(seed)
+    heads, dim = [(8, 128), (4, 256), (16, 64), (2, 8), (3, 16), (32, 32), (1, 128)][rng.integers(7)]
+    seq = int(rng.choice([32, 64, 256, 1024]))
+    batch, layers = int(rng.integers(1, 5)), int(rng.integers(1, 6))
+    ring = bool(rng.integers(2))
+    quantized = bool(rng.integers(2))
+    prompt = int(rng.choice([p for p in (8, 16, 24, 40, 64, 128) if p <= seq]))
+    seq_len = int(rng.integers(1, prompt + 1))
+    slot = int(rng.integers(batch))
+    current_position = int(rng.integers(seq)) if ring else 0
+    scale_dtype = torch.float32 if (quantized and rng.integers(2)) else torch.bfloat16
+    print(f"seed {seed} ring {ring} quantized {quantized} batch {batch} heads {heads} seq {seq} dim {dim} "
+          f"layers {layers} prompt {prompt} seq_len {seq_len} slot {slot} pos {current_position} {scale_dtype}", flush=True)
+    run_both(ring, quantized, (batch, heads, seq, dim, layers), prompt=prompt, seq_len=seq_len, slot=slot,
+             current_position=current_position, scale_dtype=scale_dtype)
