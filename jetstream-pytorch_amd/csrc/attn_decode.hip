@@ -260,8 +260,8 @@ bool attn_fast_supported(const jpt_attn_args& a, AttnMode mode) {
   if (a.k_scale && (!aligned(a.k_scale, 16) || !aligned(a.v_scale, 16))) return false;
   if (!aligned(a.q, 16) || !aligned(a.k, 16) || !aligned(a.v, 16)) return false;
   if (a.new_k && (!aligned(a.new_k, 16) || !aligned(a.new_v, 16))) return false;
-  // the new token's raw rows of all heads must fit a tile's key area
-  if (a.new_k_raw && (a.kv_heads > 16 || !aligned(a.new_k_raw, 16) || !aligned(a.new_v_raw, 16))) return false;
+  // the new token's raw rows of all heads must fit a tile (its key and value areas together)
+  if (a.new_k_raw && (a.kv_heads > 32 || !aligned(a.new_k_raw, 16) || !aligned(a.new_v_raw, 16))) return false;
   return true;
 }
 

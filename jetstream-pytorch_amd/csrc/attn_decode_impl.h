@@ -372,6 +372,9 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   const bool has_new = a.new_k != nullptr;
   // the new token arrives unquantised: the consumer of its tile quantises it
   const bool quant_new = std::is_same<KV, int8_t>::value && a.new_k_raw != nullptr;
+  // more than 16 KV heads: the token's raw rows fill two tiles, keys then values,
+  // each spread over the key and the value area; one consumer takes both
+  const bool wide_new = quant_new && a.kv_heads > 16;
   // the new token is also written into its slot's page (paged caches)
   const bool to_pages = PAGED && has_new && a.new_to_pages != 0;
 
@@ -449,7 +452,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   // empty slot is an inactive one and has no token)
   auto cache_tiles = [&](const Item& it) { return (it.count + kTile - 1) / kTile; };
   auto item_tiles = [&](const Item& it) {
-    return cache_tiles(it) + ((has_new && it.start == 0 && !(to_pages && it.len == 0)) ? 1 : 0);
+    return cache_tiles(it) + ((has_new && it.start == 0 && !(to_pages && it.len == 0)) ? (wide_new ? 2 : 1) : 0);
   };
   // Bounded wait for an LDS counter; false = give up (abort raised).
   auto wait_for = [&](int* counter, int needed) -> bool {
@@ -592,7 +595,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     // the key/value areas receive the first bytes at tk/tv as they lie (the new
     // token's unquantised rows) instead of `valid` swizzled rows.
     auto issue_tile = [&](const char* tk, const char* tv, const char* sc, const float* mk, int valid,
-                          bool raw) -> bool {
+                          bool raw, int raw_k_pieces = 0, int raw_v_pieces = 0) -> bool {
       JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
       JPT_TR(if (tr_line && issued < 256) tr_line[issued * 8 + 0] = tr_t;)
       if (!wait_counter(&sm_freed[fill_slot], fill_round, C::kLoadsPerTile)) return false;
@@ -603,9 +606,11 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       if (raw) {
 #pragma unroll
         for (int j = 0; j < kLoadsPerMatrix; ++j) {
-          const uint32_t off = static_cast<uint32_t>(min(64 * j + lane, a.kv_heads * (kD / 8) - 1)) * 16;
-          __builtin_amdgcn_global_load_lds((global_ptr)(tk + off), (lds_ptr)(slot + j * 1024), 16, 0, 0);
-          __builtin_amdgcn_global_load_lds((global_ptr)(tv + off), (lds_ptr)(slot + C::kTileBytes + j * 1024), 16, 0, 0);
+          // 16-byte pieces of the rows, clamped to those there are
+          const uint32_t off_k = static_cast<uint32_t>(min(64 * j + lane, raw_k_pieces - 1)) * 16;
+          const uint32_t off_v = static_cast<uint32_t>(min(64 * j + lane, raw_v_pieces - 1)) * 16;
+          __builtin_amdgcn_global_load_lds((global_ptr)(tk + off_k), (lds_ptr)(slot + j * 1024), 16, 0, 0);
+          __builtin_amdgcn_global_load_lds((global_ptr)(tv + off_v), (lds_ptr)(slot + C::kTileBytes + j * 1024), 16, 0, 0);
         }
       } else {
 #pragma unroll
@@ -703,7 +708,14 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         const char* sc = scale_lane;
         if (SCALE == kScaleF32) sc = new_scale_lane + (static_cast<int64_t>(cur.slot) * a.scale_heads + hs) * kEs;
         const float* mk = MASK ? static_cast<const float*>(a.mask) + cur.slot * a.mask_stride_b : nullptr;
-        if (!issue_tile(tk, tv, sc, mk, 1, quant_new)) return;
+        const int pieces = a.kv_heads * (kD / 8);  // of one raw tensor's rows
+        if (wide_new) {
+          constexpr int kAreaPieces = C::kTileBytes / 16;
+          if (!issue_tile(tk, tk + C::kTileBytes, sc, mk, 1, true, kAreaPieces, pieces - kAreaPieces)) return;
+          if (!issue_tile(tv, tv + C::kTileBytes, sc, mk, 1, true, kAreaPieces, pieces - kAreaPieces)) return;
+        } else if (!issue_tile(tk, tv, sc, mk, 1, quant_new, pieces, pieces)) {
+          return;
+        }
       }
       for (int ct = 0; ct < n_cache; ++ct) {
         const int t0 = cur.start + ct * kTile;
@@ -877,7 +889,16 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     if (quant_here) {
       const float* rope = a.new_k_rope ? a.new_k_rope + static_cast<int64_t>(cur_slot) * kD : nullptr;
       float k0, k1, v0, v1;
-      const float mk = new_absmax(slot, rope, k0, k1), mv = new_absmax(slot + C::kTileBytes, nullptr, v0, v1);
+      // the raw value rows: this tile's value area, or all of the next tile
+      const char* v_rows = slot + C::kTileBytes;
+      const int s2 = (t + 1) % C::kSlots;
+      if (wide_new) {
+        if (!wait_for(&sm_filled[s2], (t + 1) / C::kSlots + 1)) return false;
+        v_rows = ring + s2 * C::kSlotBytes;
+      }
+      const float mk = new_absmax(slot, rope, k0, k1), mv = new_absmax(v_rows, nullptr, v0, v1);
+      if (wide_new && lane == 0)  // the next tile has been read (the release waits for the reads)
+        __hip_atomic_fetch_add(&sm_freed[s2], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
       const float rk = row_max(mk), rv = row_max(mv);  // both reductions in flight together
       new_ks = new_encode(slot, static_cast<int8_t*>(const_cast<void*>(a.new_k)), const_cast<void*>(a.new_k_scale), k0, k1,
                           rows_max(rk));
@@ -1179,6 +1200,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     l_run = 0.f;
     // this consumer's tiles: stream numbers congruent to its index
     for (int ti = (wave + kConsumers - base % kConsumers) % kConsumers; ti < nt; ti += kConsumers) {
+      if (wide_new && ti == 1 && nt - n_cache == 2) continue;  // read by the consumer of tile 0
       const bool is_new = ti < nt - n_cache;  // the new token comes first
       const int valid = is_new ? 1 : min(kTile, cur.count - (ti - (nt - n_cache)) * kTile);
       if (valid == kTile) {

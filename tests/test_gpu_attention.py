@@ -240,8 +240,8 @@ def test_fused_new_token_equals_unfused_and_concatenation(quantized):
 def test_attention_launch_quantises_the_new_token(rounding, sdt, per_head, hq, hkv, d):
   """new_key_raw: the attention launch does the quantiser's work too.  Codes
   and scales must be the separate quantiser's bit for bit (which the oracle
-  pins), the output that of attending those codes.  32 KV heads and head_dim
-  64 take the library's quantise-first route."""
+  pins), the output that of attending those codes.  Head_dim 64 takes the
+  library's quantise-first route."""
   from jetstream_pt_amd import attention_kernel as ak
   from jetstream_pt_amd.quantize import quantize_kv
   from oracle import quant as oq
@@ -267,7 +267,13 @@ def test_attention_launch_quantises_the_new_token(rounding, sdt, per_head, hq, h
                               new_rounding=rounding)
   assert torch.equal(nk, wk) and torch.equal(nv, wv), "codes"
   assert torch.equal(nks, wks) and torch.equal(nvs, wvs), "scales"
-  assert torch.equal(got, want) and torch.equal(m, wm) and torch.equal(l, wl)
+  if hkv <= 16 or d != 128:
+    assert torch.equal(got, want) and torch.equal(m, wm) and torch.equal(l, wl)
+  else:
+    # more than 16 KV heads: the raw token takes two tiles, so the cache tiles fall to
+    # other consumers than in the launch that is given the codes - another summation order
+    check_out(got.reshape(b, hq, 1, d), want.reshape(b, hq, 1, d).float().cpu(), "32 KV heads")
+    assert torch.allclose(m, wm, rtol=STAT_RTOL, atol=1e-4) and torch.allclose(l, wl, rtol=STAT_RTOL)
 
 
 @pytest.mark.parametrize("kind", ["bf16", "int8", "tiny_f32"])
