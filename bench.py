@@ -302,9 +302,10 @@ def build_paged(torch, args, int8):
         pam.free_pages_resource_many(dslots)
         pam.reserve_pages_insert_many(dslots, dns)
         dlens.index_copy_(0, dslots.long(), dns)
-        for slot, n in zip(slots, ns):
-          ids = pam.page_indices[int(slot), : (int(n) + ps - 1) // ps]  # device view: no copy
-          gins.insert_prefix_pages_int8_stacked(prompt_k[:, :, :n], prompt_v[:, :, :n], pools_k, pools_v, sk, sv, ids)
+        # all of the step's prompts in one launch; page ids are views of the device table (no copy)
+        gins.insert_prompts_pages_int8_stacked(
+            [(prompt_k[:, :, :n], prompt_v[:, :, :n]) for n in ns], pools_k, pools_v, sk, sv,
+            [pam.page_indices[int(slot), : (int(n) + ps - 1) // ps] for slot, n in zip(slots, ns)])
         if log_on:
           state["log"].append(("free_many", slots.copy()))
           state["log"].append(("insert_many", slots.copy(), ns.copy(),

@@ -247,6 +247,28 @@ int32_t jpt_prefill_insert_layers(const jpt_prefill_insert_args* args,
                                   const jpt_insert_layer* layers,
                                   int32_t n_layers, void* stream);
 
+/* Several prompts into the pages of one pool in one launch (the engine's
+ * insert, engine.py:583-626, for every request whose prefill has finished).
+ * `args` gives the destination (dst_k/dst_v/k_scale/v_scale, stacked layers by
+ * n_layers and the dst/scale layer strides), geometry, dtypes and rounding; its
+ * source, page_ids, tokens and n_pages fields are ignored.  `prompts` is a HOST
+ * array: per prompt the source (heads, tokens, dim) tensors, their strides in
+ * elements (src_head_stride 0 = tokens * dim), the DEVICE array of its n_pages
+ * page ids and its token count.  Equivalent to one jpt_prefill_insert a prompt
+ * (and done that way for shapes the one-launch kernel does not take: it
+ * needs bf16 prompts, int8 pages, heads * dim == 1024). */
+typedef struct {
+  const void* src_k;
+  const void* src_v;
+  const int32_t* page_ids;
+  int64_t src_head_stride, src_layer_stride;
+  int32_t tokens, n_pages;
+} jpt_insert_prompt;
+
+int32_t jpt_prefill_insert_prompts(const jpt_prefill_insert_args* args,
+                                   const jpt_insert_prompt* prompts,
+                                   int32_t n_prompts, void* stream);
+
 /* ------------------------------------------------------------------------
  * Decode attention.
  *

@@ -181,23 +181,16 @@ __global__ void __launch_bounds__(256) prefill_insert_kernel(InsertParams p) {
 // pass and the quantise pass, so the prompt is read once, in wide loads that
 // are all issued before the first wait.  Same op order as the general kernel.
 constexpr int kTokensPerBlock = 8;
+// Tokens t0 .. t0 + 7 of the prompt `a` describes (tokens, page_ids, n_pages,
+// src_head_stride), read from src, written to dst / scale_out.
 template <bool BF16_MATH>
-__global__ void __launch_bounds__(256) prefill_insert_quant4_kernel(InsertParams p) {
-  const jpt_prefill_insert_args& a = p.a;
+__device__ __forceinline__ void quant_insert_tokens(const jpt_prefill_insert_args& a, const uint16_t* src, char* dst,
+                                                    void* scale_out, int t0) {
   constexpr int kPasses = kTokensPerBlock / 2;
   const int half = threadIdx.x >> 7;  // which of the pass's two tokens
-  const int t0 = blockIdx.x * kTokensPerBlock;
-  const bool is_v = blockIdx.y == 1;
-  const int layer = blockIdx.z;
   const bool paged = a.page_ids != nullptr;
   const int H = a.heads, D = a.dim;
   const int rows = paged ? a.n_pages * a.page_size : a.tokens;
-  const int esz_scale = a.scale_dtype == JPT_F32 ? 4 : 2;
-  const void* src_any;
-  char* dst;
-  void* scale_out;
-  layer_tensors(p, layer, is_v, 2, 1, esz_scale, &src_any, &dst, &scale_out);
-  const uint16_t* src = static_cast<const uint16_t*>(src_any);
   const int i0 = 8 * (threadIdx.x & 127), h = i0 / D, d = i0 - h * D;
   const int groups = a.scale_heads;
   const int64_t head_stride = a.src_head_stride > 0 ? a.src_head_stride : static_cast<int64_t>(a.tokens) * D;
@@ -298,6 +291,47 @@ __global__ void __launch_bounds__(256) prefill_insert_quant4_kernel(InsertParams
       store_from_f32(scale_out, idx, a.scale_dtype, s);
     }
   }
+}
+
+template <bool BF16_MATH>
+__global__ void __launch_bounds__(256) prefill_insert_quant4_kernel(InsertParams p) {
+  const jpt_prefill_insert_args& a = p.a;
+  const bool is_v = blockIdx.y == 1;
+  const void* src;
+  char* dst;
+  void* scale_out;
+  layer_tensors(p, blockIdx.z, is_v, 2, 1, a.scale_dtype == JPT_F32 ? 4 : 2, &src, &dst, &scale_out);
+  quant_insert_tokens<BF16_MATH>(a, static_cast<const uint16_t*>(src), dst, scale_out, blockIdx.x * kTokensPerBlock);
+}
+
+// Several prompts into the pages of one stacked pool in one launch: the
+// workgroups of all prompts side by side (prompt r owns those from
+// first_block[r] on), layers along z by the layer strides.
+constexpr int kLaunchPrompts = 32;
+struct PromptsParams {
+  jpt_prefill_insert_args a;  // destination, geometry, dtypes; its source and page fields are unused
+  int32_t n_prompts;
+  int32_t first_block[kLaunchPrompts + 1];
+  jpt_insert_prompt prompt[kLaunchPrompts];
+};
+
+template <bool BF16_MATH>
+__global__ void __launch_bounds__(256) prefill_insert_prompts_kernel(PromptsParams p) {
+  int r = 0;
+  while (r + 1 < p.n_prompts && static_cast<int>(blockIdx.x) >= p.first_block[r + 1]) ++r;
+  const jpt_insert_prompt& pr = p.prompt[r];
+  jpt_prefill_insert_args a = p.a;
+  a.tokens = pr.tokens;
+  a.n_pages = pr.n_pages;
+  a.page_ids = pr.page_ids;
+  a.src_head_stride = pr.src_head_stride;
+  const bool is_v = blockIdx.y == 1;
+  const int layer = blockIdx.z;
+  const uint16_t* src = static_cast<const uint16_t*>(is_v ? pr.src_v : pr.src_k) + layer * pr.src_layer_stride;
+  char* dst = static_cast<char*>(is_v ? a.dst_v : a.dst_k) + layer * a.dst_layer_stride;
+  const int esz_scale = a.scale_dtype == JPT_F32 ? 4 : 2;
+  void* scale_out = static_cast<char*>(is_v ? a.v_scale : a.k_scale) + layer * a.scale_layer_stride * esz_scale;
+  quant_insert_tokens<BF16_MATH>(a, src, dst, scale_out, (static_cast<int>(blockIdx.x) - p.first_block[r]) * kTokensPerBlock);
 }
 
 }  // namespace
@@ -405,6 +439,67 @@ int32_t jpt_prefill_insert_layers(const jpt_prefill_insert_args* args, const jpt
   for (int32_t l0 = 0; l0 < n_layers; l0 += kTableLayers) {
     const int32_t n = n_layers - l0 < kTableLayers ? n_layers - l0 : kTableLayers;
     const int32_t st = insert_launch(*args, layers + l0, n, stream);
+    if (st != JPT_OK) return st;
+  }
+  return JPT_OK;
+}
+
+int32_t jpt_prefill_insert_prompts(const jpt_prefill_insert_args* args, const jpt_insert_prompt* prompts,
+                                   int32_t n_prompts, void* stream) {
+  using namespace jpt;
+  JPT_REQUIRE(args != nullptr && prompts != nullptr, "NULL argument");
+  JPT_REQUIRE(n_prompts >= 1, "n_prompts must be positive");
+  const jpt_prefill_insert_args& a = *args;
+  const int n_layers = a.n_layers > 0 ? a.n_layers : 1;
+  const int d8 = a.dim / 8;
+  // the shape the one-launch kernel takes; anything else goes prompt by prompt
+  bool wide = a.dst_dtype == JPT_I8 && a.in_dtype == JPT_BF16 && a.heads * a.dim == 1024 && a.dim % 8 == 0 &&
+              a.heads > 0 && (a.scale_heads == 1 || (a.scale_heads == a.heads && d8 <= 64 && (d8 & (d8 - 1)) == 0)) &&
+              a.dst_k && a.dst_v && a.k_scale && a.v_scale && aligned(a.dst_k, 8) && aligned(a.dst_v, 8) &&
+              a.dst_layer_stride % 8 == 0 && a.total_pages > 0 && a.page_size > 0 && n_layers <= 65535 &&
+              (a.scale_dtype == JPT_BF16 || a.scale_dtype == JPT_F32) &&
+              (a.rounding == JPT_ROUND_TRUNC || a.rounding == JPT_ROUND_RNE);
+  for (int32_t r = 0; r < n_prompts && wide; ++r) {
+    const jpt_insert_prompt& pr = prompts[r];
+    wide = pr.src_k && pr.src_v && pr.page_ids && pr.tokens > 0 && pr.n_pages > 0 &&
+           static_cast<int64_t>(pr.n_pages) * a.page_size >= pr.tokens && aligned(pr.src_k, 16) &&
+           aligned(pr.src_v, 16) && pr.src_layer_stride % 8 == 0 &&
+           (pr.src_head_stride == 0 || (pr.src_head_stride % 8 == 0 &&
+                                        pr.src_head_stride >= static_cast<int64_t>(pr.tokens) * a.dim));
+  }
+  if (!wide) {
+    for (int32_t r = 0; r < n_prompts; ++r) {
+      jpt_prefill_insert_args one = a;
+      one.src_k = prompts[r].src_k;
+      one.src_v = prompts[r].src_v;
+      one.page_ids = prompts[r].page_ids;
+      one.tokens = prompts[r].tokens;
+      one.n_pages = prompts[r].n_pages;
+      one.src_head_stride = prompts[r].src_head_stride;
+      one.src_layer_stride = prompts[r].src_layer_stride;
+      const int32_t st = insert_launch(one, nullptr, 0, stream);
+      if (st != JPT_OK) return st;
+    }
+    return JPT_OK;
+  }
+  for (int32_t r0 = 0; r0 < n_prompts; r0 += kLaunchPrompts) {
+    PromptsParams p{};
+    p.a = a;
+    p.a.n_layers = n_layers;
+    p.n_prompts = n_prompts - r0 < kLaunchPrompts ? n_prompts - r0 : kLaunchPrompts;
+    int blocks = 0;
+    for (int r = 0; r < p.n_prompts; ++r) {
+      p.prompt[r] = prompts[r0 + r];
+      p.first_block[r] = blocks;
+      blocks += (prompts[r0 + r].n_pages * a.page_size + kTokensPerBlock - 1) / kTokensPerBlock;
+    }
+    p.first_block[p.n_prompts] = blocks;
+    const dim3 grid(blocks, 2, n_layers);
+    if (a.scale_dtype == JPT_BF16)
+      hipLaunchKernelGGL(prefill_insert_prompts_kernel<true>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    else
+      hipLaunchKernelGGL(prefill_insert_prompts_kernel<false>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    const int32_t st = launch_status("prefill_insert_prompts_kernel");
     if (st != JPT_OK) return st;
   }
   return JPT_OK;

@@ -88,6 +88,11 @@ class InsertLayer(_c.Structure):
               ("k_scale", _vp), ("v_scale", _vp)]
 
 
+class InsertPrompt(_c.Structure):
+  _fields_ = [("src_k", _vp), ("src_v", _vp), ("page_ids", _vp), ("src_head_stride", _i64),
+              ("src_layer_stride", _i64), ("tokens", _i32), ("n_pages", _i32)]
+
+
 class AttnArgs(_c.Structure):
   _fields_ = [
       ("q", _vp), ("k", _vp), ("v", _vp), ("k_scale", _vp), ("v_scale", _vp),
@@ -125,6 +130,7 @@ _sig("jpt_paged_gather", _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_paged_append_quant_i8", _i32, _c.POINTER(PagedQuantAppendArgs), _vp)
 _sig("jpt_prefill_insert", _i32, _c.POINTER(PrefillInsertArgs), _vp)
 _sig("jpt_prefill_insert_layers", _i32, _c.POINTER(PrefillInsertArgs), _c.POINTER(InsertLayer), _i32, _vp)
+_sig("jpt_prefill_insert_prompts", _i32, _c.POINTER(PrefillInsertArgs), _c.POINTER(InsertPrompt), _i32, _vp)
 _sig("jpt_attn_workspace_bytes", _i64, _c.POINTER(AttnArgs))
 _sig("jpt_attn_plan", _i32, _c.POINTER(AttnArgs), _i32, _vp)
 _sig("jpt_attn_ragged", _i32, _c.POINTER(AttnArgs), _vp)
@@ -157,7 +163,7 @@ EXPORTS = (
     "jpt_pam_fill_new_pages", "jpt_pam_page_token_indices", "jpt_pam_free",
     "jpt_pam_free_count", "jpt_paged_append_dev", "jpt_dpam_init", "jpt_dpam_reserve_insert",
     "jpt_dpam_free", "jpt_dpam_decode_step", "jpt_decode_advance", "jpt_rope",
-    "jpt_ragged_block_indices", "jpt_prefill_insert_layers",
+    "jpt_ragged_block_indices", "jpt_prefill_insert_layers", "jpt_prefill_insert_prompts",
 )
 
 

@@ -168,6 +168,38 @@ def insert_prefix_pages_int8_stacked(prefix_k, prefix_v, pages_k, pages_v, k_sca
   _ffi.check(_ffi.lib.jpt_prefill_insert(a, _ffi.stream()))
 
 
+def insert_prompts_pages_int8_stacked(prefixes, pages_k, pages_v, k_scale_pages, v_scale_pages, page_ids, *,
+                                      rounding="rne"):
+  """Several prompts at once, all layers, one launch: prefixes is a list of
+  (prefix_k, prefix_v) pairs, each (L, heads, T_i, D); page_ids a list of
+  int32 device tensors (prompt i's pages, e.g. rows of the device allocator's
+  table).  Same result as insert_prefix_pages_int8_stacked once a prompt."""
+  pk, pv = _ffi.dev(pages_k, "pages_k"), _ffi.dev(pages_v, "pages_v")
+  ks, vs = _ffi.dev(k_scale_pages, "k_scale_pages"), _ffi.dev(v_scale_pages, "v_scale_pages")
+  layers, heads, total, ps, dim = pk.shape
+  recs, keep = [], []
+  for (newk, newv), ids in zip(prefixes, page_ids):
+    if not (newk.is_cuda and newk.stride(3) == 1 and newk.stride(2) == newk.shape[3] and
+            newk.stride() == newv.stride()):
+      newk, newv = _ffi.dev(newk.contiguous(), "prefix key"), _ffi.dev(newv.contiguous(), "prefix value")
+    if newk.shape[0] != layers or newk.shape[1] != heads or newk.shape[3] != dim or newk.dtype != prefixes[0][0].dtype:
+      raise ValueError(f"prefix {tuple(newk.shape)} does not match pages {tuple(pk.shape)}")
+    ids = _ffi.as_i32(ids, pk.device)
+    recs.append(_ffi.InsertPrompt(_ffi.ptr(newk), _ffi.ptr(newv), _ffi.ptr(ids), newk.stride(1), newk.stride(0),
+                                  newk.shape[2], ids.numel()))
+    keep += [newk, newv, ids]
+  if not recs:
+    return
+  a = _ffi.PrefillInsertArgs(
+      dst_k=_ffi.ptr(pk), dst_v=_ffi.ptr(pv), k_scale=_ffi.ptr(ks), v_scale=_ffi.ptr(vs), heads=heads, dim=dim,
+      total_pages=total, page_size=ps, in_dtype=_ffi.dtype_code(prefixes[0][0].dtype), dst_dtype=_ffi.I8,
+      scale_dtype=_ffi.dtype_code(ks.dtype), scale_heads=ks.shape[1], rounding=_rounding_code(rounding),
+      n_layers=layers, dst_layer_stride=pk.stride(0), scale_layer_stride=ks.stride(0))
+  table = (_ffi.InsertPrompt * len(recs))(*recs)
+  _ffi.check(_ffi.lib.jpt_prefill_insert_prompts(a, table, len(recs), _ffi.stream()))
+  del keep
+
+
 def insert(env, prefix_caches, prefix_seq_len, caches, cache_scales, slot, *, current_position=0,
            mask=None, start=None, input_pos=None, lens=None):
   """The reference's Engine.insert for dense caches: picks no-wrap or wrap as

@@ -181,3 +181,37 @@ def test_random_dense_inserts(block):
           f"layers {layers} prompt {prompt} seq_len {seq_len} slot {slot} pos {current_position} {scale_dtype}", flush=True)
     run_both(ring, quantized, (batch, heads, seq, dim, layers), prompt=prompt, seq_len=seq_len, slot=slot,
              current_position=current_position, scale_dtype=scale_dtype)
+
+
+@pytest.mark.parametrize("heads,dim", [(8, 128), (2, 8)])
+def test_int8_paged_insert_of_several_prompts_in_one_launch(heads, dim):
+  """Prompts of different lengths into one stacked pool with one call: the
+  pool must equal prompt-by-prompt inserts bit for bit.  (8, 128) takes the
+  one-launch kernel, (2, 8) the library's prompt-by-prompt route."""
+  import numpy as np
+  from jetstream_pt_amd import insert as gins
+  layers, total, ps = 3, 40, 32
+  g = torch.Generator().manual_seed(9)
+  rng = np.random.default_rng(9)
+  pk = torch.randint(-127, 128, (layers, heads, total, ps, dim), generator=g, dtype=torch.int8)
+  pv = torch.randint(-127, 128, (layers, heads, total, ps, dim), generator=g, dtype=torch.int8)
+  sk, sv = torch.rand((layers, 1, total, ps), generator=g), torch.rand((layers, 1, total, ps), generator=g)
+  lens = [1, 33, 64, 100, 7, 160]
+  perm = rng.permutation(total).astype(np.int32)
+  buf_k = torch.randn((layers, heads, 200, dim), generator=g).to(torch.bfloat16).to(DEV)  # one long buffer, prompts are its heads
+  buf_v = torch.randn((layers, heads, 200, dim), generator=g).to(torch.bfloat16).to(DEV)
+  prefixes, ids, at = [], [], 0
+  for n in lens:
+    need = -(-n // ps)
+    ids.append(torch.from_numpy(perm[at:at + need].copy()).to(DEV))
+    at += need
+    prefixes.append((buf_k[:, :, :n], buf_v[:, :, :n]))
+  many = [t.to(DEV) for t in (pk, pv, sk, sv)]
+  one = [t.to(DEV) for t in (pk, pv, sk, sv)]
+  gins.insert_prompts_pages_int8_stacked(prefixes, *many, ids)
+  for (k, v), i in zip(prefixes, ids):
+    gins.insert_prefix_pages_int8_stacked(k, v, *one, i)
+  torch.cuda.synchronize()
+  for a, b in zip(many, one):
+    assert torch.equal(a, b)
+  assert not torch.equal(many[0].cpu(), pk)
