@@ -12,6 +12,13 @@ a stacked cache (64 GiB of codes), so every step streams cold data; once per
 32 steps the per-step split plan is recomputed and finalize() scatters the 32
 stashed tokens into the cache (both inside the timed region).
 
+Timing: a pass over the layers (plan, every layer's step, finalize) is
+captured once in a HIP graph and replayed at least 50 times, each replay
+between its own pair of events on the stream the work runs on; `ms_per_step`
+is the MEDIAN replay divided by the layers in it, `min_us_per_layer` the
+fastest, `repeats` the number of replays (`steps`/`warmup` echo the command
+line: enough whole passes are run to cover them).
+
 Prints one JSON line.  `value` is algorithmic bytes of the layer-step divided
 by its time; `roofline` is the attention launch alone (a separate timed loop
 of attention launches only); `cpu_baseline` times the CPU oracle's
@@ -21,11 +28,13 @@ The other configurations of BASELINE.json are parity-test cases; `--workload
 c1|c2|c4|c5` times them the same way for the record (same JSON shape, no
 cpu_baseline):
   c1  dense bf16 eager update + dense attention, B=8, 32 heads, S=1024
-  c2  int8 MHA decode step, B=96, 32 heads, S=2048, lengths U[128, 2048]
+  c2  int8 MHA decode step, B=96, 32 heads, S=2048, lengths U[128, 2048] (a slot at
+      2048 is full: it is attended, its new token is attended too but not stored)
   c4  paged bf16, B=256, 64 q / 8 kv heads, 32768 pages of 64, page
       allocation every decode step, paged attention that appends the token
   c5  paged int8, 32 layers, B=256, 32 q / 8 kv heads, 16384 pages of 64 per
-      layer; every decode step frees 16 slots and inserts 16 new prompts
+      layer; every decode step frees 16 slots and inserts 16 new prompts;
+      a slot that has reached max_cache_len (4096) retires before the step
 """
 
 import argparse
@@ -45,11 +54,24 @@ D = 128
 B, HQ, HKV, S, LAYERS = 128, 32, 8, 8192, 32  # the headline workload
 SEED = 3
 PROBE_COPY_BYTES = 1 << 30
-# HBM bytes of one attention launch (decode kernel + merge kernel) on the
-# headline workload, from hardware counters (FETCH_SIZE + WRITE_SIZE, each
-# calibrated on a 1 GiB copy; see --probe-traffic).  A recorded measurement,
-# not computed here.
-MEASURED_ATTN_TRAFFIC_BYTES = 157_450_000
+# HBM bytes of one attention launch on the headline workload, from hardware
+# counters (FETCH_SIZE + WRITE_SIZE, each calibrated on a 1 GiB copy; see
+# --probe-traffic): a recorded measurement, kept in the summary of the counter
+# runs under profiles/ and read from there.
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "attn_decode_c3_int8_hbm_traffic_pmc.txt")
+MIN_REPEATS = 50
+
+
+def measured_attn_traffic_bytes():
+  """The `traffic_bytes_per_launch:` line of the counter summary, or None."""
+  try:
+    with open(TRAFFIC_SUMMARY) as f:
+      for line in f:
+        if line.startswith("traffic_bytes_per_launch:"):
+          return int(line.split(":")[1].split()[0])
+  except (OSError, ValueError):
+    pass
+  return None
 DEV = "cuda:0"
 
 
@@ -95,6 +117,7 @@ def build_dense_int8(torch, nl, batch, hq, hkv, seq, lengths, name):
   from jetstream_pt_amd.environment import JetEngineEnvironment, JetEngineEnvironmentData
 
   env = JetEngineEnvironment(JetEngineEnvironmentData(batch_size=batch, num_layers=nl, ring_buffer=False))
+  torch.manual_seed(SEED)  # the cache contents below come from the device's default generator
   cache = cm.Int8KVCacheGenerate.empty((nl, batch, hkv, seq, D), DEV, env, scale_heads=1,
                                        scale_dtype=torch.float32)
   for l in range(nl):  # codes uniform [-127, 127], scales U(0.005, 0.05)
@@ -152,11 +175,13 @@ def build_c3(torch, args):
 
 
 def build_c2(torch, args):
-  lengths = uniform_lengths(torch, 96, 128, 2047, seed=2)
+  lengths = uniform_lengths(torch, 96, 128, 2048, seed=2)
+  if getattr(args, "full_slot", False):  # parity tests: the edge of the range, whatever the draw holds
+    lengths[0] = 2048
   w = build_dense_int8(torch, args.layers or 32, 96, 32, 32, 2048, lengths,
                        "C2 int8 MHA decode layer-step: KV quantise+stash, ragged attention with fused new "
                        "token, finalize amortised over the layers")
-  w["config"]["lengths"] = "uniform [128, 2047], seed 2"
+  w["config"]["lengths"] = "uniform [128, 2048], seed 2"
   return w
 
 
@@ -232,13 +257,14 @@ def build_paged(torch, args, int8):
   log_on = bool(getattr(args, "log", host_alloc))  # index arrays kept for the parity tests
   if int8:
     nl, batch, hq, hkv, ps, total, max_pages, seed = args.layers or 32, 256, 32, 8, 64, 16384, 64, 5
-    lengths = seeded_lengths(torch, batch, 600.0, 16, 4096 - 256, seed).numpy().astype(np.int32)
+    lengths = seeded_lengths(torch, batch, 600.0, 16, 4096, seed).numpy().astype(np.int32)
   else:
     nl, batch, hq, hkv, ps, total, max_pages, seed = args.layers or 4, 256, 64, 8, 64, 32768, 128, 4
     lengths = uniform_lengths(torch, batch, 32, 2048, seed).numpy().astype(np.int32)
   env = JetEngineEnvironment(JetEngineEnvironmentData(
       batch_size=batch, num_layers=nl, paged_attention_total_num_pages=total, paged_attention_page_size=ps))
   rng = np.random.default_rng(seed)
+  torch.manual_seed(seed)  # pool contents come from the device's default generator
   order = rng.permutation(total).astype(np.int32)
   if host_alloc:
     pam = PageAttentionManager(batch, total, ps, max_pages, free_list_order=order)
@@ -287,6 +313,18 @@ def build_paged(torch, args, int8):
     prompts take over some slots, then (host allocator only) pages for the
     step are reserved and the tables uploaded.  Also the byte accounting."""
     lens = state["lens"]
+    full = np.nonzero(lens >= max_pages * ps)[0].astype(np.int32)
+    if len(full):  # a slot at max_cache_len cannot take another token: its request is over, the slot retires
+      if host_alloc:
+        for slot in full:
+          pam.free_pages_resource(int(slot))
+      else:
+        dfull = to_dev_async(full)
+        pam.free_pages_resource_many(dfull)
+        dlens.index_fill_(0, dfull.long(), 0)
+      if log_on:
+        state["log"].append(("free_many", full.copy()))
+      lens[full] = 0
     if churn:
       slots = rng.choice(batch, churn, replace=False).astype(np.int32)
       ns = np.array([int(rng.integers(64, 1025)) for _ in slots], dtype=np.int32)
@@ -394,10 +432,12 @@ def run_gpu(args):
   use_graph = w["graph"] and not args.no_graph
 
   def timed(fn, steps, warmup, before=None):
-    """fn(i) enqueues step i.  Whole passes over the layers are replayed from
-    one captured HIP graph where the workload allows (what a serving loop does
-    with a launch-bound decode step); a remainder of steps from a shorter one.
-    before(), when given, is the eager per-pass work ahead of layer 0."""
+    """fn(i) enqueues step i.  A whole pass over the layers is replayed from one
+    captured HIP graph where the workload allows (what a serving loop does with
+    a launch-bound decode step), otherwise launched from Python.  before(),
+    when given, is the eager per-pass work ahead of layer 0 (it is inside the
+    timed region).  Every pass is timed by its own pair of events; returns
+    (median, min, mean over the whole region) in ms per step and the passes."""
     before = before or (lambda: None)
     warmup = (max(warmup, nl) + nl - 1) // nl * nl  # whole passes
     for i in range(warmup):
@@ -405,47 +445,37 @@ def run_gpu(args):
         before()
       fn(i)
     torch.cuda.synchronize()
-    graph = rest = None
+    graph = None
     if use_graph:
-      def capture(n):
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-          for i in range(n):
-            fn(i)
-        before()
-        g.replay()
-        torch.cuda.synchronize()
-        return g
-      if steps >= nl:
-        graph = capture(nl)
-      if steps % nl:  # the steps left over after the whole passes: a shorter graph of their own
-        rest = capture(steps % nl)
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    done = 0
-    if graph is not None:
-      for _ in range(steps // nl):
-        before()
-        graph.replay()
-      done = steps // nl * nl
-    if rest is not None:
+      graph = torch.cuda.CUDAGraph()
+      with torch.cuda.graph(graph):
+        for i in range(nl):
+          fn(i)
       before()
-      rest.replay()
-      done = steps
-    for i in range(done, steps):
-      if i % nl == 0:
-        before()
-      fn(i)
-    stop.record()
+      graph.replay()
+      torch.cuda.synchronize()
+    passes = max((steps + nl - 1) // nl, MIN_REPEATS)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(passes + 1)]
+    marks[0].record()
+    for r in range(passes):
+      before()
+      if graph is not None:
+        graph.replay()
+      else:
+        for i in range(nl):
+          fn(i)
+      marks[r + 1].record()
     torch.cuda.synchronize()
-    return start.elapsed_time(stop) / steps
+    each = sorted(marks[r].elapsed_time(marks[r + 1]) / nl for r in range(passes))
+    whole = marks[0].elapsed_time(marks[passes]) / (passes * nl)
+    return each[len(each) // 2], each[0], whole, passes
 
-  ms_per_step = timed(w["step"], args.steps, args.warmup, w.get("before_pass"))
+  ms_per_step, ms_min, ms_mean, passes = timed(w["step"], args.steps, args.warmup, w.get("before_pass"))
   if "bytes_now" in w:
     w["step_bytes"], w["attn_bytes"] = w["bytes_now"]()
-  attn_ms = timed(w["attn_only"], args.steps, args.warmup)
-  w.update(ms_per_step=ms_per_step, attn_ms=attn_ms, launch="hip graph of one pass over the layers" if use_graph
-           else "python")
+  attn_ms, attn_min, _, _ = timed(w["attn_only"], args.steps, args.warmup)
+  w.update(ms_per_step=ms_per_step, ms_min=ms_min, ms_mean=ms_mean, repeats=passes, attn_ms=attn_ms,
+           attn_min=attn_min, launch="hip graph of one pass over the layers" if use_graph else "python")
   return w
 
 
@@ -591,14 +621,19 @@ def main():
       "data": "synthetic",
       "config": cfg,
       "us_per_layer": round(r["ms_per_step"] * 1e3, 2),
+      "min_us_per_layer": round(r["ms_min"] * 1e3, 2),
+      "mean_us_per_layer": round(r["ms_mean"] * 1e3, 2),
+      "repeats": r["repeats"],
+      "timing": f"median of {r['repeats']} passes over {cfg['layers_rotated']} layers, each pass between its own events",
       "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 1),
       "tokens_per_s": round(cfg["batch"] / (r["ms_per_step"] * 1e-3 * model_layers), 1),
       "roofline": {
           "bound": "hbm", "kernel": r["kernel"],
           "achieved": round(attn_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
           "frac": round(attn_gbps / HBM_PEAK_GBPS, 4),
-          "traffic": MEASURED_ATTN_TRAFFIC_BYTES if headline and cfg["layers_rotated"] == LAYERS else None,
-          "us_per_launch": round(r["attn_ms"] * 1e3, 2), "algorithmic_bytes": int(r["attn_bytes"]),
+          "traffic": measured_attn_traffic_bytes() if headline and cfg["layers_rotated"] == LAYERS else None,
+          "us_per_launch": round(r["attn_ms"] * 1e3, 2), "min_us_per_launch": round(r["attn_min"] * 1e3, 2),
+          "algorithmic_bytes": int(r["attn_bytes"]),
       },
   }
   if first_use is not None:

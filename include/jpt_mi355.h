@@ -131,7 +131,8 @@ int32_t jpt_rope(void* out, const void* x, const float* freqs, int32_t rows,
  *   pages[h, page_j, tok_j, :] = src[slot_j, h, 0, :]; src is
  *   (batch, heads, 1, row_bytes).
  * jpt_paged_gather   - PageAttentionManager._compress_cache (:195-200):
- *   dst[h, t, :] = pages[h, page_row[t / ps], t % ps, :] for t < length.
+ *   dst[h, t, :] = pages[h, page_row[t / ps], t % ps, :] for t < length;
+ *   page_row holds max_pages ids, and length <= max_pages * ps is required.
  * `page_ids`, `indices`, `page_row` are int32 device arrays.
  * ---------------------------------------------------------------------- */
 int32_t jpt_paged_insert(void* pages_k, void* pages_v, const void* src_k,
@@ -156,8 +157,9 @@ int32_t jpt_paged_append_dev(void* pages_k, void* pages_v, const void* src_k,
                              int32_t page_size, int32_t row_bytes, void* stream);
 
 int32_t jpt_paged_gather(void* dst, const void* pages, const int32_t* page_row,
-                         int32_t length, int32_t heads, int32_t total_pages,
-                         int32_t page_size, int32_t row_bytes, void* stream);
+                         int32_t max_pages, int32_t length, int32_t heads,
+                         int32_t total_pages, int32_t page_size,
+                         int32_t row_bytes, void* stream);
 
 /* int8 pages (no reference counterpart: the reference's paged cache is
  * bf16/f32 only, cache_manager.py:717-724).  Same row scatter as
@@ -325,25 +327,37 @@ int32_t jpt_prefill_insert_prompts(const jpt_prefill_insert_args* args,
  * multiple of 32); other shapes are refused.
  *
  * workspace: device scratch of at least jpt_attn_workspace_bytes(args)
- * bytes, 256-byte aligned.  Its first JPT_ATTN_WS_STATE_BYTES must be zero
- * before the first call and are left zero by every call; calls sharing one
- * workspace must not overlap in time.
+ * bytes, 256-byte aligned.  Its first JPT_ATTN_WS_STATE_BYTES (the state
+ * block) must be zero before the first call; calls sharing one workspace
+ * must not overlap in time.
+ *
+ * Errors.  Shape and state errors are refused before anything is enqueued
+ * (JPT_E_BADARG; the reference raises on them, attention_kernel.py:525-526,
+ * :547-550).  Every wait inside the streaming kernel is bounded; a wave whose
+ * wait runs out gives up, the launch ends, and word 0 of the state block is
+ * set and stays set: what the launch wrote is then not to be used.  The launch
+ * itself cannot report this (the call only enqueues); jpt_attn_status does.
  * ---------------------------------------------------------------------- */
 #define JPT_ATTN_WS_STATE_BYTES 65536
+#define JPT_ATTN_STATUS_GAVE_UP 1
+#define JPT_ATTN_STATUS_SLOT_FULL 2
 
 typedef struct {
   const void* q;
-  const void* k;
-  const void* v;
-  const void* k_scale;
-  const void* v_scale;
+  /* k, v and their scales are read-only, except with new_to_pages, which writes
+   * the new token's row and scales into them; new_k/new_v and their scales are
+   * inputs, except with new_k_raw, which makes them outputs: hence no const */
+  void* k;
+  void* v;
+  void* k_scale;
+  void* v_scale;
   const int32_t* lengths;
   const int32_t* page_table;
   const void* mask;
-  const void* new_k;
-  const void* new_v;
-  const void* new_k_scale;
-  const void* new_v_scale;
+  void* new_k;
+  void* new_v;
+  void* new_k_scale;
+  void* new_v_scale;
   void* out;
   float* out_max;
   float* out_denom;
@@ -383,6 +397,19 @@ int32_t jpt_attn_plan(const jpt_attn_args* args, int32_t paged, void* stream);
 int32_t jpt_attn_ragged(const jpt_attn_args* args, void* stream);
 int32_t jpt_attn_dense(const jpt_attn_args* args, void* stream);
 int32_t jpt_attn_paged(const jpt_attn_args* args, void* stream);
+/* Waits for `stream`, then stores the workspace's status word into *status
+ * and clears it.  Bits, sticky since the last call:
+ *   JPT_ATTN_STATUS_GAVE_UP    a launch gave up (see Errors above);
+ *   JPT_ATTN_STATUS_SLOT_FULL  a plan saw a slot whose length had reached the
+ *     cache capacity (seq, or max_pages * page_size): the slot is attended up
+ *     to the capacity, and a token appended to it in that step is attended
+ *     but NOT stored (every append on this path skips positions outside the
+ *     cache; the reference's dynamic_update_slice would clamp the position
+ *     and overwrite the last row, cache_manager.py:154-173).
+ *  Synchronises: call it where the caller synchronises anyway (the
+ * reference raises from inside its jitted step; a kernel cannot).  Not to be
+ * called during stream capture. */
+int32_t jpt_attn_status(void* workspace, void* stream, int32_t* status);
 
 /* Log-sum-exp merge of two partial attention results (layers.py:539-548):
  * out = (l1*a*o1 + b*o2*l2) / (a*l1 + b*l2), a = exp(m1-g), b = exp(m2-g),

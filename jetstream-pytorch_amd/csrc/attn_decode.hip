@@ -15,7 +15,6 @@
 // len * 128 * (bytes(K) + bytes(V)) plus len * (bytes(k_scale) +
 // bytes(v_scale)) / heads-sharing-a-scale.
 #include <math.h>
-#include <stdlib.h>
 
 #include "attn_common.h"
 #include "attn_plan.h"
@@ -27,7 +26,8 @@ constexpr int kChunkAlign = 128;
 constexpr float kLn2 = 0.6931471805599453f;
 
 // ---- workspace layout --------------------------------------------------------
-// [0, 64 KiB)   reserved state block (kept zero)
+// [0, 64 KiB)   state block, zero before the first call; word 0 is the sticky
+//               give-up flag that jpt_attn_status reads and clears
 // then          sorted plan entries, per-slot chunk table, partials
 struct Layout {
   int64_t entries, slots, partials, total;
@@ -37,33 +37,22 @@ struct Layout {
 constexpr int kMaxPlanBatch = 4096;
 constexpr int kMaxChunksPerSlot = 256;
 
-int32_t env_int(const char* name, int32_t fallback) {
-  const char* e = getenv(name);
-  const int32_t t = e ? atoi(e) : 0;
-  return t > 0 ? t : fallback;
-}
-
-int32_t persistent_blocks();
-
-// Work items (chunk x KV head) the planner aims for: five for every four
-// workers.  An item costs a few microseconds beyond its tiles (query rows,
-// fold, output or partial), so chunks are made about as long as a worker's
-// share of the positions, and the sort-and-deal of the plan evens out the rest.
-int32_t target_items() {
-  static int32_t v = env_int("JPT_ATTN_TARGET_ITEMS", persistent_blocks() * 5 / 4);
-  return v;
-}
-
+// Workers of the streaming kernel: two groups of waves on every compute unit.
 int32_t persistent_blocks() {
   static int32_t v = [] {
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) == hipSuccess)
       if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cus = 256;
-    const int32_t per_cu = env_int("JPT_ATTN_BLOCKS_PER_CU", 2);
-    return (cus * per_cu + 7) / 8 * 8;
+    return (cus * 2 + 7) / 8 * 8;
   }();
   return v;
 }
+
+// Work items (chunk x KV head) the planner aims for: five for every four
+// workers.  An item costs a few microseconds beyond its tiles (query rows,
+// fold, output or partial), so chunks are made about as long as a worker's
+// share of the positions, and the sort-and-deal of the plan evens out the rest.
+int32_t target_items() { return persistent_blocks() * 5 / 4; }
 
 Layout make_layout(int batch, int kv_heads, int rows) {
   Layout l;
@@ -108,7 +97,7 @@ __device__ __forceinline__ int plan_exclusive_scan(int x, int* total) {
 
 __global__ void __launch_bounds__(256)
 plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int target,
-            PlanEntry* entries, SlotChunks* slots, int max_entries) {
+            PlanEntry* entries, SlotChunks* slots, int max_entries, int32_t* status) {
   __shared__ int s_len[kMaxPlanBatch];
   __shared__ int s_first[kMaxPlanBatch];
   __shared__ long long s_total;
@@ -120,12 +109,15 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
   for (int i = tid; i < 257; i += blockDim.x) s_hist[i] = 0;
   __syncthreads();
   long long mine = 0;
+  bool full = false;  // a slot with no room left for the step's token
   for (int b = tid; b < batch; b += blockDim.x) {
     int n = lengths ? lengths[b] : seq_cap;
+    full = full || (lengths && n >= seq_cap);
     n = n < 0 ? 0 : (n > seq_cap ? seq_cap : n);
     s_len[b] = n;
     mine += n;
   }
+  if (full) atomicOr(status, JPT_ATTN_STATUS_SLOT_FULL);
   atomicAdd(reinterpret_cast<unsigned long long*>(&s_total), static_cast<unsigned long long>(mine));
   __syncthreads();
   if (tid == 0) {
@@ -267,23 +259,27 @@ bool attn_fast_supported(const jpt_attn_args& a, AttnMode mode) {
 
 int64_t attn_fast_workspace_bytes(const jpt_attn_args& a) {
   const int rows = a.q_heads / a.kv_heads * a.q_rows;
+  // shapes the streaming kernel never takes (prefill-shaped queries, huge
+  // batches) run on the generic kernel, which uses neither plan nor partials
+  if (rows > kMaxRows || a.batch > kMaxPlanBatch) return JPT_ATTN_WS_STATE_BYTES;
   return make_layout(a.batch, a.kv_heads, rows).total;
 }
 
 int32_t attn_plan_launch(const jpt_attn_args& a, bool paged, hipStream_t stream) {
   const int rows = a.q_heads / a.kv_heads * a.q_rows;
+  if (rows > kMaxRows || a.batch > kMaxPlanBatch) return JPT_OK;  // generic kernel: nothing to plan
   const Layout l = make_layout(a.batch, a.kv_heads, rows);
   JPT_REQUIRE(a.workspace != nullptr && a.workspace_bytes >= l.total,
               "workspace of %lld bytes needed, %lld given", static_cast<long long>(l.total),
               static_cast<long long>(a.workspace_bytes));
   JPT_REQUIRE(aligned(a.workspace, 256), "workspace must be 256-byte aligned");
-  JPT_REQUIRE(a.batch <= kMaxPlanBatch, "batch above %d", kMaxPlanBatch);
   char* ws = static_cast<char*>(a.workspace);
   const int cap = paged ? a.max_pages * a.page_size : a.seq;
   JPT_REQUIRE(cap > 0, "sequence capacity must be positive");
   hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(256), 0, stream, a.lengths, a.batch, cap,
                      a.kv_heads, target_items(), reinterpret_cast<PlanEntry*>(ws + l.entries),
-                     reinterpret_cast<SlotChunks*>(ws + l.slots), l.max_entries);
+                     reinterpret_cast<SlotChunks*>(ws + l.slots), l.max_entries,
+                     reinterpret_cast<int32_t*>(ws));
   return launch_status("plan_kernel");
 }
 
@@ -304,12 +300,7 @@ int32_t attn_fast_launch(const jpt_attn_args& a, AttnMode mode, hipStream_t stre
   p.rows = rows;
   p.rep = rep;
   p.total_items = l.max_entries * a.kv_heads;
-#ifdef JPT_ATTN_TRACE
-  {
-    const char* e = getenv("JPT_TRACE_PTR");
-    p.trace = e ? reinterpret_cast<unsigned long long*>(strtoull(e, nullptr, 0)) : nullptr;
-  }
-#endif
+  p.status = reinterpret_cast<int32_t*>(ws);
   if (!a.reuse_plan) {
     int32_t st = attn_plan_launch(a, mode == kPaged, stream);
     if (st != JPT_OK) return st;
@@ -349,10 +340,10 @@ static int32_t attn_entry(const jpt_attn_args* args, jpt::AttnMode mode, void* s
     jpt_quant_append_args q{};
     q.new_k = a.new_k_raw;
     q.new_v = a.new_v_raw;
-    q.out_k = const_cast<void*>(a.new_k);
-    q.out_v = const_cast<void*>(a.new_v);
-    q.out_k_scale = const_cast<void*>(a.new_k_scale);
-    q.out_v_scale = const_cast<void*>(a.new_v_scale);
+    q.out_k = a.new_k;
+    q.out_v = a.new_v;
+    q.out_k_scale = a.new_k_scale;
+    q.out_v_scale = a.new_v_scale;
     q.batch = a.batch;
     q.heads = a.kv_heads;
     q.dim = a.dim;
@@ -378,6 +369,21 @@ int32_t jpt_attn_plan(const jpt_attn_args* args, int32_t paged, void* stream) {
   JPT_REQUIRE(args->batch > 0 && args->kv_heads > 0 && args->q_heads > 0 && args->q_rows > 0 &&
                   args->q_heads % args->kv_heads == 0, "batch, heads and q_rows must be positive");
   return attn_plan_launch(*args, paged != 0, static_cast<hipStream_t>(stream));
+}
+
+int32_t jpt_attn_status(void* workspace, void* stream, int32_t* status) {
+  using namespace jpt;
+  JPT_REQUIRE(workspace != nullptr && status != nullptr, "workspace and status must not be NULL");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int32_t word = 0;
+  JPT_HIP(hipMemcpyAsync(&word, workspace, sizeof(word), hipMemcpyDeviceToHost, s));
+  JPT_HIP(hipStreamSynchronize(s));
+  if (word != 0) {
+    JPT_HIP(hipMemsetAsync(workspace, 0, sizeof(word), s));
+    JPT_HIP(hipStreamSynchronize(s));
+  }
+  *status = word;
+  return JPT_OK;
 }
 
 int32_t jpt_attn_ragged(const jpt_attn_args* args, void* stream) { return attn_entry(args, jpt::kRagged, stream); }

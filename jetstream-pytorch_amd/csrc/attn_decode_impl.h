@@ -13,10 +13,12 @@
 //                   contiguous cache rows; a first touch of a new cache row
 //                   (several microseconds with its TLB miss) is hidden behind
 //                   the tiles already in the ring.
-//   consumer waves  take tiles round-robin out of the ring, convert int8 codes
-//                   to bf16 in registers (exact) and run
-//                       S^T = K . Q^T   v_mfma_f32_16x16x32_bf16, positions on
-//                                       M, the rep*q_rows query rows on N
+//   consumer waves  take tiles round-robin out of the ring, turn int8 codes
+//                   into float16 operands with byte permutes (exact; bf16
+//                   caches go in as they are) and run
+//                       S^T = K . Q^T   v_mfma_f32_16x16x32_f16 / _bf16,
+//                                       positions on M, the rep*q_rows query
+//                                       rows on N
 //                       O^T = V^T . P^T positions on the contraction index
 //                   with an online softmax in between.  The score
 //                   accumulators of lane (row r, group g) are exactly the
@@ -30,8 +32,10 @@
 // over through LDS counters, and the consumer that delivers the last part of an
 // item folds the parts and writes the slot's output (one chunk) or parks the
 // chunk's float32 partial (several; a second kernel folds those).  Every wait
-// is bounded: a wave that waits too long raises an abort flag and every wave
-// leaves, so a logic error shows up as wrong output, never as a hung GPU.
+// is bounded: a wave that waits too long raises an abort flag, every wave of
+// the workgroup leaves, and a sticky word in the workspace's state block tells
+// the host that the launch's results are not to be used (jpt_attn_status), so
+// a logic error shows up as an error, never as a hung GPU.
 #pragma once
 
 #include <math.h>
@@ -52,24 +56,9 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef const __attribute__((address_space(1))) void* global_ptr;
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
-#ifndef JPT_ATTN_EXPERIMENT_CUT
-// Development builds for timing experiments only (results are wrong): 1, 2 stop a
-// tile's work early; 3 skips an item's fold and output; 4 only the fold by the
-// last consumer to arrive; 5 the conversion of the query operand; 6 the fold's
-// global stores.
-#define JPT_ATTN_EXPERIMENT_CUT 0
-#endif
-#ifndef JPT_ATTN_CONSUMERS
-#define JPT_ATTN_CONSUMERS 3
-#endif
-#ifndef JPT_ATTN_GROUPS
-#define JPT_ATTN_GROUPS 2
-#endif
-#ifndef JPT_ATTN_WAVES_PER_SIMD
-#define JPT_ATTN_WAVES_PER_SIMD 2
-#endif
-constexpr int kConsumers = JPT_ATTN_CONSUMERS;
-constexpr int kGroups = JPT_ATTN_GROUPS;
+constexpr int kConsumers = 3;
+constexpr int kGroups = 2;
+constexpr int kWavesPerSimd = 2;
 constexpr int kGroupWaves = kConsumers + 1;  // wave 0 of a group is its producer
 constexpr int kWaves = kGroups * kGroupWaves;
 constexpr int kThreads = kWaves * 64;
@@ -308,13 +297,6 @@ struct Tile<__bf16> {
   __device__ __forceinline__ static Op ones() { return as_op<Op>(0, 0, 0, 0); }  // unused
 };
 
-// Per-wave timing records for development builds (-DJPT_ATTN_TRACE): eight
-// 64-bit words per wave, times in ticks of the 100 MHz real-time counter.
-#ifdef JPT_ATTN_TRACE
-#define JPT_TR(stmt) stmt
-#else
-#define JPT_TR(stmt)
-#endif
 
 // One work item: a chunk of one slot for one KV head.
 struct Item {
@@ -324,7 +306,7 @@ struct Item {
 };
 
 template <typename KV, bool PAGED, int SCALE, bool MASK, int RC>
-__global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode_kernel(FastParams p) {
+__global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(FastParams p) {
   using C = Config<KV, SCALE, MASK, RC>;
   const jpt_attn_args& a = p.a;
   __shared__ __attribute__((aligned(1024))) char ring_all[kGroups][C::kSlots * C::kSlotBytes];
@@ -338,7 +320,6 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   __shared__ int sm_arrived_all[kGroups][C::kFoldBufs];
   __shared__ int sm_folded_all[kGroups][C::kFoldBufs];
   __shared__ int sm_abort;
-  JPT_TR(__shared__ int sm_issue_time[kGroups][C::kSlots];)
   __shared__ __attribute__((aligned(16))) int sm_items_all[kGroups][kListedItems][8];
   // page ids of the item being issued and of the next one (paged caches)
   __shared__ int sm_pages_all[PAGED ? kGroups : 1][2][kStagedPages];
@@ -348,10 +329,6 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   const int group = hw_wave / kGroupWaves;
   // role index: consumers 0..kConsumers-1, producer kConsumers
   const int wave = hw_wave % kGroupWaves == 0 ? kConsumers : hw_wave % kGroupWaves - 1;
-  JPT_TR(const unsigned long long tr_start = __builtin_amdgcn_s_memrealtime();)
-  JPT_TR(unsigned long long* tr_line = (p.trace && blockIdx.x == 5 && group == 0 && lane == 0) ? p.trace + 1024 * 16 * 8 : nullptr;)
-  JPT_TR(unsigned long long tr_sig = 0; int tr_polls = 0; unsigned long long tr_qwait = 0;)
-  JPT_TR(unsigned long long tr_wait = 0; unsigned long long tr_fold = 0; unsigned long long tr_first = 0; unsigned long long tr_t = 0; int tr_tiles = 0;)
   for (int i = tid; i < kGroups * C::kSlots; i += kThreads) {
     (&sm_filled_all[0][0])[i] = 0;
     (&sm_freed_all[0][0])[i] = 0;
@@ -454,13 +431,20 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   auto item_tiles = [&](const Item& it) {
     return cache_tiles(it) + ((has_new && it.start == 0 && !(to_pages && it.len == 0)) ? (wide_new ? 2 : 1) : 0);
   };
+  // A wave gives up: the other waves of the workgroup see the flag at their
+  // next wait and leave too, and the host finds the sticky word in the
+  // workspace's state block (jpt_attn_status).
+  auto give_up = [&]() {
+    lds_poke(&sm_abort, 1);
+    if (lane == 0) __hip_atomic_fetch_or(p.status, JPT_ATTN_STATUS_GAVE_UP, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
   // Bounded wait for an LDS counter; false = give up (abort raised).
   auto wait_for = [&](int* counter, int needed) -> bool {
     int spins = 0;
     while (__hip_atomic_load(counter, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < needed) {
       if (++spins > kSpinLimit ||
           __hip_atomic_load(&sm_abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) {
-        __hip_atomic_store(&sm_abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        give_up();
         return false;
       }
       __builtin_amdgcn_s_sleep(1);
@@ -518,8 +502,6 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
                          (PAGED ? static_cast<int>((carries_p >> (signalled & 63)) & 1) : 0);
         if (done < need) break;
         lds_poke(&sm_filled[sig_slot], sig_round);  // every lane stores the same word
-        JPT_TR(tr_fold += static_cast<unsigned>(static_cast<int>(__builtin_amdgcn_s_memrealtime()) - lds_peek(&sm_issue_time[group][sig_slot]));)
-        JPT_TR(if (tr_line && signalled < 256) tr_line[signalled * 8 + 2] = __builtin_amdgcn_s_memrealtime();)
         sig_base = need;
         carries_q &= ~(1ull << (signalled & 63));
         if (PAGED) carries_p &= ~(1ull << (signalled & 63));
@@ -531,12 +513,10 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     // `room` more loads fit under the load counter's limit of 63.
     auto wait_counter = [&](int* counter, int needed, int room) -> bool {
       for (int spins = 0;; ++spins) {
-        JPT_TR(const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();)
         signal_landed();
-        JPT_TR(tr_sig += __builtin_amdgcn_s_memrealtime() - t0; ++tr_polls;)
         if (loads_issued - sig_base + room <= 63 && lds_peek_uniform(counter) >= needed) return true;
         if (spins > kSpinLimit || lds_peek_uniform(&sm_abort)) {
-          lds_poke(&sm_abort, 1);
+          give_up();
           __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
           return false;
         }
@@ -552,7 +532,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         const int out = static_cast<int>((ib & 0xF) | (((ib >> 22) & 0x3) << 4));
         if (loads_issued - out >= target && loads_issued - sig_base + room <= 63) return true;
         if (spins > kSpinLimit || lds_peek_uniform(&sm_abort)) {
-          lds_poke(&sm_abort, 1);
+          give_up();
           __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
           return false;
         }
@@ -596,13 +576,8 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     // token's unquantised rows) instead of `valid` swizzled rows.
     auto issue_tile = [&](const char* tk, const char* tv, const char* sc, const float* mk, int valid,
                           bool raw, int raw_k_pieces = 0, int raw_v_pieces = 0) -> bool {
-      JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
-      JPT_TR(if (tr_line && issued < 256) tr_line[issued * 8 + 0] = tr_t;)
       if (!wait_counter(&sm_freed[fill_slot], fill_round, C::kLoadsPerTile)) return false;
-      JPT_TR(if (tr_line && issued < 256) tr_line[issued * 8 + 1] = __builtin_amdgcn_s_memrealtime();)
-      JPT_TR(tr_wait += __builtin_amdgcn_s_memrealtime() - tr_t; if (!tr_first) tr_first = __builtin_amdgcn_s_memrealtime() - tr_start;)
       char* slot = ring + fill_slot * C::kSlotBytes;
-      JPT_TR(lds_poke(&sm_issue_time[group][fill_slot], static_cast<int>(__builtin_amdgcn_s_memrealtime()));)
       if (raw) {
 #pragma unroll
         for (int j = 0; j < kLoadsPerMatrix; ++j) {
@@ -748,17 +723,12 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     for (int spins = 0; signalled < issued; ++spins) {
       signal_landed();
       if (spins > kSpinLimit || lds_peek_uniform(&sm_abort)) {
-        lds_poke(&sm_abort, 1);
+        give_up();
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
         return;
       }
       __builtin_amdgcn_s_sleep(1);
     }
-    JPT_TR(if (p.trace && lane == 0) {
-      unsigned long long* o = p.trace + (static_cast<size_t>(blockIdx.x) * kWaves + hw_wave) * 8;
-      o[0] = issued; o[1] = tr_wait; o[2] = tr_fold; o[3] = __builtin_amdgcn_s_memrealtime() - tr_start;
-      o[4] = tr_start; o[5] = 0; o[6] = tr_first; o[7] = (static_cast<unsigned long long>(tr_polls) << 32) | tr_sig;
-    })
     return;
   }
 
@@ -874,14 +844,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   auto consume_tile = [&](int t, int valid, bool is_new, auto full_tag) -> bool {
     constexpr bool FULL = decltype(full_tag)::value;
     const int s = t % C::kSlots;
-    JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
     if (!wait_for(&sm_filled[s], t / C::kSlots + 1)) return false;
-    JPT_TR(tr_wait += __builtin_amdgcn_s_memrealtime() - tr_t; ++tr_tiles; if (!tr_first) tr_first = __builtin_amdgcn_s_memrealtime() - tr_start;)
-#ifdef JPT_ATTN_EXPERIMENT_NO_COMPUTE
-    if (lane == 0)
-      __hip_atomic_fetch_add(&sm_freed[s], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
-    return true;
-#endif
     char* slot = ring + s * C::kSlotBytes;
     const char* side = slot + 2 * C::kTileBytes;
     float new_ks = 0.f, new_vs = 0.f;
@@ -900,10 +863,10 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       if (wide_new && lane == 0)  // the next tile has been read (the release waits for the reads)
         __hip_atomic_fetch_add(&sm_freed[s2], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
       const float rk = row_max(mk), rv = row_max(mv);  // both reductions in flight together
-      new_ks = new_encode(slot, static_cast<int8_t*>(const_cast<void*>(a.new_k)), const_cast<void*>(a.new_k_scale), k0, k1,
+      new_ks = new_encode(slot, static_cast<int8_t*>(a.new_k), a.new_k_scale, k0, k1,
                           rows_max(rk));
-      new_vs = new_encode(slot + C::kTileBytes, static_cast<int8_t*>(const_cast<void*>(a.new_v)),
-                          const_cast<void*>(a.new_v_scale), v0, v1, rows_max(rv));
+      new_vs = new_encode(slot + C::kTileBytes, static_cast<int8_t*>(a.new_v),
+                          a.new_v_scale, v0, v1, rows_max(rv));
     }
     T tile;
     tile.read(slot, slot + C::kTileBytes, r, g, pos);
@@ -964,31 +927,12 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     if (lane == 0)
       __hip_atomic_fetch_add(&sm_freed[s], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
 
-#if JPT_ATTN_EXPERIMENT_CUT == 1
-    {
-      uint32_t keep = 0;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) keep ^= tile.v[i].x ^ tile.v[i].y;
-      keep ^= tile.ka[0].x ^ tile.ka[1].w ^ tile.kb[0].y ^ tile.kb[1].z ^ __float_as_uint(ks[0] + vs[7]);
-      asm volatile("" ::"v"(keep));
-      return true;
-    }
-#endif
     f32x4 sa = s_init, sb = s_init;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
       sa = T::mfma(tile.k_op(false, kk), qop[kk], sa);
       sb = T::mfma(tile.k_op(true, kk), qop[kk], sb);
     }
-#if JPT_ATTN_EXPERIMENT_CUT == 2
-    {
-      uint32_t keep = 0;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) keep ^= tile.v[i].x ^ tile.v[i].y;
-      asm volatile("" ::"v"(keep), "v"(sa), "v"(sb), "v"(ks[0] + vs[7]));
-      return true;
-    }
-#endif
     float sc[8];
     float tmax = -INFINITY;
 #pragma unroll
@@ -1031,9 +975,6 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
   // consumer to arrive folds the parts and writes the slot's output (one
   // chunk) or parks the chunk's partial (several).
   auto finish_item = [&](const Item& it, int seq) -> bool {
-#if JPT_ATTN_EXPERIMENT_CUT == 3
-    return true;
-#endif
     const int buf = seq % C::kFoldBufs;
     // the buffer's previous item must have been folded out of it
     if (!wait_for(&sm_folded[buf], seq / C::kFoldBufs)) return false;
@@ -1055,13 +996,6 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
       arrived = __hip_atomic_fetch_add(&sm_arrived[buf], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_WORKGROUP);
     arrived = __builtin_amdgcn_readfirstlane(arrived);
     if (arrived != kConsumers - 1) return true;
-#if JPT_ATTN_EXPERIMENT_CUT == 4
-    if (lane == 0) {
-      __hip_atomic_store(&sm_arrived[buf], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      __hip_atomic_fetch_add(&sm_folded[buf], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
-    }
-    return true;
-#endif
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     const int64_t q_row0 = (static_cast<int64_t>(it.slot) * a.q_heads + it.h * p.rep) * a.q_rows;
     float* part = p.partials + (static_cast<int64_t>(it.part) * a.kv_heads + it.h) * R * kPartFloats;
@@ -1083,10 +1017,6 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         o[0] += x.x * f; o[1] += x.y * f; o[2] += x.z * f; o[3] += x.w * f;
         o[4] += y.x * f; o[5] += y.y * f; o[6] += y.z * f; o[7] += y.w * f;
       }
-#if JPT_ATTN_EXPERIMENT_CUT == 6
-      asm volatile("" ::"v"(o[0] + o[1] + o[2] + o[3] + o[4] + o[5] + o[6] + o[7] + l + M));
-      continue;
-#endif
       if (it.n_chunks == 1) {
         const float inv = l > 0.f ? 1.f / l : 0.f;
         const uint4 packed = make_uint4(pack_bf16(o[0] * inv, o[1] * inv), pack_bf16(o[2] * inv, o[3] * inv),
@@ -1129,9 +1059,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     const int n_cache = cache_tiles(cur), nt = item_tiles(cur);
     if (nt > 0) {
       // query rows: staged by the producer ahead of the item's first tile
-      JPT_TR(const unsigned long long tq0 = __builtin_amdgcn_s_memrealtime();)
       if (!wait_for(&sm_filled[base % C::kSlots], base / C::kSlots + 1)) return;
-      JPT_TR(tr_qwait += __builtin_amdgcn_s_memrealtime() - tq0;)
       const int qb = q_seq++ % C::kQBufs;
       uint4 u[4];
 #pragma unroll
@@ -1139,7 +1067,7 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         u[kk] = make_uint4(0, 0, 0, 0);
         if (r < R) u[kk] = *reinterpret_cast<const uint4*>(&sm_q[qb][r][32 * g + 8 * kk]);
       }
-      if (T::kBias == 0.f || JPT_ATTN_EXPERIMENT_CUT == 5) {
+      if (T::kBias == 0.f) {
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) qop[kk] = __builtin_bit_cast(Op, u[kk]);
       } else {
@@ -1211,12 +1139,12 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
     }
     if (keep) {  // this consumer had the new token's tile
       keep = false;
-      if (dst_room) {
-        const int page = min(max(dst_page, 0), a.total_pages - 1);  // whatever the table holds, stay inside the pool
+      if (dst_room && dst_page >= 0) {  // a negative id: the allocator had no page for this token
+        const int page = min(dst_page, a.total_pages - 1);  // whatever the table holds, stay inside the pool
         const int64_t in_pool = static_cast<int64_t>(page) * a.page_size + cur.len % a.page_size;
         const int64_t row = static_cast<int64_t>(cur.h) * a.total_pages * a.page_size + in_pool;
-        char* dk = static_cast<char*>(const_cast<void*>(a.k)) + row * C::kRowBytes + lane * kLaneBytes;
-        char* dv = static_cast<char*>(const_cast<void*>(a.v)) + row * C::kRowBytes + lane * kLaneBytes;
+        char* dk = static_cast<char*>(a.k) + row * C::kRowBytes + lane * kLaneBytes;
+        char* dv = static_cast<char*>(a.v) + row * C::kRowBytes + lane * kLaneBytes;
         if (kLaneBytes == 2) {
           *reinterpret_cast<uint16_t*>(dk) = static_cast<uint16_t>(keep_k);
           *reinterpret_cast<uint16_t*>(dv) = static_cast<uint16_t>(keep_v);
@@ -1226,21 +1154,14 @@ __global__ void __launch_bounds__(kThreads, JPT_ATTN_WAVES_PER_SIMD) attn_decode
         }
         if (SCALE && lane == 0 && (a.scale_heads != 1 || cur.h == 0)) {
           const int64_t si = static_cast<int64_t>(a.scale_heads == 1 ? 0 : cur.h) * a.total_pages * a.page_size + in_pool;
-          store_from_f32(const_cast<void*>(a.k_scale), si, kBf16Math ? JPT_BF16 : JPT_F32, keep_ks);
-          store_from_f32(const_cast<void*>(a.v_scale), si, kBf16Math ? JPT_BF16 : JPT_F32, keep_vs);
+          store_from_f32(a.k_scale, si, kBf16Math ? JPT_BF16 : JPT_F32, keep_ks);
+          store_from_f32(a.v_scale, si, kBf16Math ? JPT_BF16 : JPT_F32, keep_vs);
         }
       }
     }
-    JPT_TR(tr_t = __builtin_amdgcn_s_memrealtime();)
     if (!finish_item(cur, seq++)) return;
-    JPT_TR(tr_fold += __builtin_amdgcn_s_memrealtime() - tr_t;)
     base += nt;
   }
-  JPT_TR(if (p.trace && lane == 0) {
-    unsigned long long* o = p.trace + (static_cast<size_t>(blockIdx.x) * kWaves + hw_wave) * 8;
-    o[0] = tr_tiles; o[1] = tr_wait; o[2] = tr_fold; o[3] = __builtin_amdgcn_s_memrealtime() - tr_start;
-    o[4] = tr_start; o[5] = seq; o[6] = tr_first; o[7] = tr_qwait;
-  })
 }
 
 // `workers` groups are wanted; a workgroup holds kGroups of them.

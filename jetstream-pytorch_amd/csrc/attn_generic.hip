@@ -57,7 +57,8 @@ __global__ void __launch_bounds__(64) attn_generic_kernel(jpt_attn_args a, int m
   // in the scale tensor.
   auto kv_row = [&](int tok, int64_t* srow) -> int64_t {
     if (paged) {
-      const int page = a.page_table[static_cast<int64_t>(b) * a.max_pages + tok / ps];
+      int page = a.page_table[static_cast<int64_t>(b) * a.max_pages + tok / ps];
+      page = min(max(page, 0), a.total_pages - 1);  // whatever the table holds, stay inside the pool
       const int64_t in_page = static_cast<int64_t>(page) * ps + tok % ps;
       *srow = static_cast<int64_t>(hs) * a.total_pages * ps + in_page;
       return static_cast<int64_t>(hkv) * a.total_pages * ps + in_page;

@@ -32,9 +32,7 @@ struct FastParams {
   int32_t rows;         // rep * q_rows
   int32_t rep;
   int32_t total_items;  // max_entries * kv_heads
-#ifdef JPT_ATTN_TRACE
-  unsigned long long* trace;  // per-wave timing records (development builds only)
-#endif
+  int32_t* status;      // word 0 of the workspace's state block: sticky, set when a wave gave up
 };
 
 namespace decode {

@@ -27,6 +27,14 @@ inline int32_t fail(int32_t code, const char* fmt, ...) {
     if (!(cond)) return jpt::fail(JPT_E_BADARG, __VA_ARGS__); \
   } while (0)
 
+// A HIP runtime call that must succeed.
+#define JPT_HIP(call)                                                            \
+  do {                                                                           \
+    hipError_t jpt_hip_e = (call);                                               \
+    if (jpt_hip_e != hipSuccess)                                                 \
+      return jpt::fail(JPT_E_HIP, "%s: %s", #call, hipGetErrorString(jpt_hip_e)); \
+  } while (0)
+
 // Checks the launch that was just enqueued.
 inline int32_t launch_status(const char* what) {
   hipError_t e = hipGetLastError();

@@ -7,7 +7,9 @@
 // ascending order, requests in the order given) without any atomics - a
 // slot's place in the hand-out order is a prefix sum over the slots before it.
 // Kernels cannot raise; a request that cannot be served is skipped and leaves
-// a bit in state[2].  No index read from memory is used before it is checked
+// a bit in state[2]; a decode step whose page request fails drops that slot's
+// token (page -1 in its column of update_indices and in its table cell)
+// instead of writing it anywhere.  No index read from memory is used before it is checked
 // against the array it addresses.
 #include <algorithm>
 
@@ -188,7 +190,10 @@ dpam_decode_step_kernel(jpt_dpam d, const int32_t* lens) {
     const int rank = popped + block_exclusive_scan(wants ? 1 : 0, &n_wants);
     const int j = active + block_exclusive_scan(len > 0 ? 1 : 0, &n_active);
     int32_t* row = d.page_indices + static_cast<int64_t>(b < d.batch ? b : 0) * d.max_pages;
-    int page = d.total_pages - 1;
+    // page = -1: the step's token of this slot has no page (a request that
+    // failed now or in an earlier step); the appends skip such a column, the
+    // table cell says so too, and the slot's length stays where it was
+    int page = -1;
     if (len > 0 && inside) page = row[p];
     if (wants) {
       if (rank < count) {
@@ -197,10 +202,13 @@ dpam_decode_step_kernel(jpt_dpam d, const int32_t* lens) {
         d.n_alloc[b] = p + 1;
       } else {
         raise(d, JPT_DPAM_NOPAGES);
+        page = -1;
+        row[p] = -1;
       }
     }
+    if (page >= d.total_pages) page = -1;
     if (b < d.batch) {
-      d.lengths[b] = len > 0 ? len + 1 : 0;
+      d.lengths[b] = len > 0 && page >= 0 ? len + 1 : len;
       if (len > 0) {
         d.update_indices[j] = page;
         d.update_indices[d.batch + j] = j * ps + len % ps;

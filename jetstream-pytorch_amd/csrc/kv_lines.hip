@@ -144,8 +144,9 @@ __global__ void __launch_bounds__(256) quant_append_kernel(QuantParams p) {
   bool write_cache = cache != nullptr;
   if (paged) {
     page = p.indices[tok];
-    at = p.indices[p.stride + tok] % p.page_size;
-    write_cache = write_cache && page >= 0 && page < p.total_pages;
+    const int tok_index = p.indices[p.stride + tok];  // j * page_size + offset in the page
+    at = tok_index % p.page_size;
+    write_cache = write_cache && page >= 0 && page < p.total_pages && tok_index >= 0;
   } else {
     at = a.pos ? a.pos[a.pos_count == 1 ? 0 : b] : 0;
     write_cache = write_cache && at >= 0 && at < a.seq;
@@ -212,8 +213,9 @@ __global__ void __launch_bounds__(256) quant_append_vec_kernel(QuantParams p) {
   bool write_cache = cache != nullptr;
   if (paged) {
     page = p.indices[tok];
-    at = p.indices[p.stride + tok] % p.page_size;
-    write_cache = write_cache && page >= 0 && page < p.total_pages;
+    const int tok_index = p.indices[p.stride + tok];  // j * page_size + offset in the page
+    at = tok_index % p.page_size;
+    write_cache = write_cache && page >= 0 && page < p.total_pages && tok_index >= 0;
   } else {
     at = a.pos ? a.pos[a.pos_count == 1 ? 0 : b] : 0;
     write_cache = write_cache && at >= 0 && at < a.seq;

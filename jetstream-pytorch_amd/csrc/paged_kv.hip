@@ -178,12 +178,15 @@ int32_t jpt_paged_append_dev(void* pages_k, void* pages_v, const void* src_k,
 }
 
 int32_t jpt_paged_gather(void* dst, const void* pages, const int32_t* page_row,
-                         int32_t length, int32_t heads, int32_t total_pages,
-                         int32_t page_size, int32_t row_bytes, void* stream) {
+                         int32_t max_pages, int32_t length, int32_t heads,
+                         int32_t total_pages, int32_t page_size,
+                         int32_t row_bytes, void* stream) {
   using namespace jpt;
   JPT_REQUIRE(dst && pages && page_row, "NULL argument");
   JPT_REQUIRE(heads > 0 && total_pages > 0 && page_size > 0 && row_bytes > 0, "heads, total_pages, page_size, row_bytes must be positive");
   JPT_REQUIRE(length >= 0, "negative length");
+  JPT_REQUIRE(max_pages > 0 && static_cast<int64_t>(length) <= static_cast<int64_t>(max_pages) * page_size,
+              "length %d is past the %d pages of the row", length, max_pages);
   if (length == 0) return JPT_OK;
   const int vec = pick_vec(row_bytes, {dst, pages});
   dim3 grid(blocks_for(static_cast<int64_t>(heads) * length * (row_bytes / vec)));

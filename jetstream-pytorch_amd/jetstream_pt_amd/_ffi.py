@@ -126,7 +126,7 @@ _sig("jpt_rope", _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_paged_insert", _i32, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_paged_append", _i32, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_paged_append_dev", _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _vp)
-_sig("jpt_paged_gather", _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp)
+_sig("jpt_paged_gather", _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp)
 _sig("jpt_paged_append_quant_i8", _i32, _c.POINTER(PagedQuantAppendArgs), _vp)
 _sig("jpt_prefill_insert", _i32, _c.POINTER(PrefillInsertArgs), _vp)
 _sig("jpt_prefill_insert_layers", _i32, _c.POINTER(PrefillInsertArgs), _c.POINTER(InsertLayer), _i32, _vp)
@@ -136,6 +136,7 @@ _sig("jpt_attn_plan", _i32, _c.POINTER(AttnArgs), _i32, _vp)
 _sig("jpt_attn_ragged", _i32, _c.POINTER(AttnArgs), _vp)
 _sig("jpt_attn_dense", _i32, _c.POINTER(AttnArgs), _vp)
 _sig("jpt_attn_paged", _i32, _c.POINTER(AttnArgs), _vp)
+_sig("jpt_attn_status", _i32, _vp, _vp, _i32p)
 _sig("jpt_lse_merge", _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _vp)
 _sig("jpt_pam_create", _i32, _i32, _i32, _i32, _i32, _i32p, _c.POINTER(_vp))
 _sig("jpt_pam_destroy", None, _vp)
@@ -164,6 +165,7 @@ EXPORTS = (
     "jpt_pam_free_count", "jpt_paged_append_dev", "jpt_dpam_init", "jpt_dpam_reserve_insert",
     "jpt_dpam_free", "jpt_dpam_decode_step", "jpt_decode_advance", "jpt_rope",
     "jpt_ragged_block_indices", "jpt_prefill_insert_layers", "jpt_prefill_insert_prompts",
+    "jpt_attn_status",
 )
 
 

@@ -2,7 +2,8 @@
 
 Same names and argument order as the reference module
 (jetstream_pt/attention_kernel.py): dense_attention (:628), flash_attention
-(:688), ragged_mha (:480), RaggedAttentionKernel (:713), call_paged_attention
+(:688), ragged_mqa (:122), ragged_mqa_reference (:342), ragged_mha (:480),
+RaggedAttentionKernel (:713), shard_kv_heads (:762), call_paged_attention
 (:789), reshape_heads / reshape_outputs (:583-602).  Tensors are torch tensors
 on the ROCm device; sharding arguments are accepted and ignored (one GPU).
 
@@ -25,7 +26,10 @@ Additions, all keyword-only or optional:
     decode step reuses one split plan instead of re-planning per layer.
 """
 
+import collections
+import ctypes
 import math
+import weakref
 
 import torch
 
@@ -36,11 +40,15 @@ from .quantize import _rounding_code
 # ---- workspace and split plans ----------------------------------------------------
 
 
+_live_workspaces = weakref.WeakSet()  # every workspace still in use, for check_status()
+
+
 class _Workspace:
   """Device scratch for the split-KV kernel; the leading state block stays zero."""
 
   def __init__(self, nbytes, device):
     self.buf = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+    _live_workspaces.add(self)
 
   @property
   def nbytes(self):
@@ -48,7 +56,42 @@ class _Workspace:
 
 
 _workspaces = {}
-_dense_workspaces = {}
+_dense_workspaces = collections.OrderedDict()  # most recently used last
+_MAX_DENSE_WORKSPACES = 8
+_FAST_MAX_ROWS = 16  # query rows per KV head (rep * T) the streaming kernel takes
+
+
+def _streaming_kernel_may_run(rows, dim, q_dtype, kv_dtype):
+  """Whether the library's streaming kernel can take this shape at all; other
+  shapes go to its shape-generic kernel, which uses no workspace and no plan."""
+  return (rows <= _FAST_MAX_ROWS and dim == 128 and q_dtype == torch.bfloat16
+          and kv_dtype in (torch.int8, torch.bfloat16))
+
+
+STATUS_GAVE_UP, STATUS_SLOT_FULL = 1, 2
+
+
+def check_status(plan=None):
+  """Raises RuntimeError if a streaming-kernel launch gave up since the last
+  check (a bounded in-kernel wait ran out: its outputs are not to be used).
+  Looks at `plan`'s workspace, or at every workspace still alive (the shared
+  ones and those of every DecodePlan).
+  Synchronises the current stream; the record is cleared by the check.
+  Returns the remaining status bits: STATUS_SLOT_FULL says that a planned step
+  saw a slot at cache capacity, whose new token was attended but not stored."""
+  if plan is not None:
+    spaces = [plan.workspace]
+  else:
+    spaces = list(_live_workspaces)
+  bad = 0
+  for ws in spaces:
+    word = ctypes.c_int32(0)
+    _ffi.check(_ffi.lib.jpt_attn_status(_ffi.ptr(ws.buf), _ffi.stream(), ctypes.byref(word)))
+    bad |= word.value
+  if bad & STATUS_GAVE_UP:
+    raise RuntimeError("a decode attention launch gave up on a bounded wait inside the kernel; "
+                       "its outputs (and any token it was to quantise or append) are not valid")
+  return bad
 
 
 def _shared_workspace(nbytes, device):
@@ -234,13 +277,17 @@ def _attend(mode, xq, keys, values, *, lengths=None, page_table=None, mask=None,
     oden = torch.empty((b, hq, t), dtype=torch.float32, device=device)
     a.out_max, a.out_denom = _ffi.ptr(omax), _ffi.ptr(oden)
 
-  if plan is not None and plan.key == (b, hq, hkv, t, a.seq or None, a.page_size or None,
-                                       a.max_pages or None) and lengths is not None \
+  ws = None
+  if not _streaming_kernel_may_run(hq // hkv * t, d, xq.dtype, keys.dtype) or force_generic:
+    pass  # prefill-shaped and other calls of the generic kernel: no workspace, no plan
+  elif plan is not None and plan.key == (b, hq, hkv, t, a.seq or None, a.page_size or None,
+                                         a.max_pages or None) and lengths is not None \
       and plan.lengths.data_ptr() == lengths.data_ptr():
     ws, a.reuse_plan = plan.workspace, 1
   elif lengths is None and mode == "dense":
     # every slot attends all `seq` positions: the split depends on the shape
-    # only, so it is planned once per (stream, shape) into a workspace of its own
+    # only, so it is planned once per (stream, shape) into a workspace of its
+    # own; the least recently used of these is dropped when there are too many
     key = (torch.device(device), torch.cuda.current_stream(device).cuda_stream, b, hq, hkv, t, a.seq)
     ws = _dense_workspaces.get(key)
     if ws is None:
@@ -250,11 +297,15 @@ def _attend(mode, xq, keys, values, *, lengths=None, page_table=None, mask=None,
       if _ffi.lib.jpt_attn_plan(pa, 0, _ffi.stream()) == _ffi.OK:
         _dense_workspaces[key] = ws
         a.reuse_plan = 1
+        while len(_dense_workspaces) > _MAX_DENSE_WORKSPACES:
+          _dense_workspaces.popitem(last=False)
     else:
+      _dense_workspaces.move_to_end(key)
       a.reuse_plan = 1
   else:
     ws = _shared_workspace(_ffi.lib.jpt_attn_workspace_bytes(a), device)
-  a.workspace, a.workspace_bytes = _ffi.ptr(ws.buf), ws.nbytes
+  if ws is not None:
+    a.workspace, a.workspace_bytes = _ffi.ptr(ws.buf), ws.nbytes
 
   fn = {"ragged": _ffi.lib.jpt_attn_ragged, "dense": _ffi.lib.jpt_attn_dense,
         "paged": _ffi.lib.jpt_attn_paged}[mode]
@@ -340,6 +391,41 @@ def ragged_mha(q, k, v, layer, start, end, ragged_batch_index=None,
   hkv = k.shape[-3]
   rows = hq // hkv * tq
   return out.reshape(bq, hkv, rows, dq), (mx.reshape(bq, hkv, rows), den.reshape(bq, hkv, rows))
+
+
+def ragged_mqa_reference(q, k, v, layer, start, end, ragged_batch_index=None,
+                         ragged_block_index=None, k_scaler=None, v_scaler=None, bk=512,
+                         mask_value=None, normalize_var=True, testing=False, quantized=False):
+  """The reference's per-KV-head entry point (attention_kernel.py:342-466), which its
+  ragged_mha vmaps over the heads: q (B, T, D); k, v (B, S, D), or stacked
+  (L, B, S, D) with `layer` picking one; scalers (B, 1, S) / (L, B, 1, S) or None.
+  Returns o (B, T, D) in q's dtype and (m, l), each (B, T) float32.  Here it is
+  ragged_mha on a single head (the launch covers all heads at once, so callers
+  with several heads should call ragged_mha)."""
+  del quantized  # told by the scalers
+  if k.dim() == 4:  # stacked
+    k, v = k[layer], v[layer]
+    if k_scaler is not None and k_scaler.dim() == 4:
+      k_scaler, v_scaler = k_scaler[layer], v_scaler[layer]
+  if q.dim() != 3 or k.dim() != 3:
+    raise ValueError(f"ragged_mqa takes q (B, T, D) and k (B, S, D); got {tuple(q.shape)}, {tuple(k.shape)}")
+  out, (m, l) = ragged_mha(q.unsqueeze(1), k.unsqueeze(1), v.unsqueeze(1), 0, start, end,
+                           ragged_batch_index, ragged_block_index, k_scaler, v_scaler, bk=bk,
+                           mask_value=mask_value, normalize_var=normalize_var, testing=testing)
+  return out.squeeze(1), (m.squeeze(1), l.squeeze(1))
+
+
+# The reference's Pallas variant of the same function (attention_kernel.py:122-252);
+# one implementation serves both names here.
+ragged_mqa = ragged_mqa_reference
+
+
+def shard_kv_heads(paged_attention_impl, mesh=None, kv_head_mesh_axis_name=None):
+  """The reference wraps its paged kernel in a shard_map over the KV heads of a
+  device mesh (attention_kernel.py:762-786).  On one GPU every head is local:
+  the function comes back as it is."""
+  del mesh, kv_head_mesh_axis_name
+  return paged_attention_impl
 
 
 class RaggedAttentionKernel:

@@ -172,7 +172,7 @@ class PageAttentionManager:
     if lens == 0:
       return out
     _ffi.check(_ffi.lib.jpt_paged_gather(
-        _ffi.ptr(out), _ffi.ptr(cache), _ffi.ptr(row), lens, heads, total, ps,
+        _ffi.ptr(out), _ffi.ptr(cache), _ffi.ptr(row), row.numel(), lens, heads, total, ps,
         dim * cache.element_size(), _ffi.stream()))
     return out
 
@@ -205,7 +205,11 @@ class DevicePageAttentionManager(PageAttentionManager):
       DeviceTokenIndices;
     * a kernel cannot raise: a request that cannot be served is skipped and
       remembered; `check()` (synchronises) raises queue.Empty / IndexError /
-      ValueError for it like the host class does at once.
+      ValueError for it like the host class does at once.  Until then
+      `reserve_pages_insert` has returned the view of the row it would have
+      filled, and a decode step has dropped the token of a slot it found no
+      page for (page id -1 in its index column and table cell; no other
+      slot's page is touched).
   """
 
   # pylint: disable-next=super-init-not-called
@@ -330,7 +334,13 @@ class DevicePageAttentionManager(PageAttentionManager):
     return int(self._state[2].item())
 
   def check(self):
+    """Raises what the host class raises at once, for every request the kernels
+    could not serve since the last check (synchronises); the record is cleared,
+    so the next check reports new failures only.  A decode step whose page
+    request failed has dropped that slot's token: nothing was written for it."""
     bits = self.status()
+    if bits:
+      self._state[2:3].zero_()
     if bits & _ffi.DPAM_NOPAGES:
       raise queue.Empty("the device free list ran out of pages")
     if bits & _ffi.DPAM_OVERFLOW:

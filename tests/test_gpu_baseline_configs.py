@@ -4,7 +4,13 @@ Each test builds the workload exactly as bench.py times it (same shapes, same
 seeded inputs, fewer layers), runs layer-steps through the product path and
 checks every byte the step writes - cache rows, codes, scales, page tables -
 bit for bit against the CPU oracle, the attention output within 1e-2, and that
-nothing else in the cache changed."""
+nothing else in the cache changed.
+
+Attention tolerance: max-abs 1e-2 against the float64 closed form rounded to the
+bf16 output, written as 1e-2 + 2^-8 |expected| (the second term is the half-ulp
+of the output's own rounding).  The oracle's restatement of the reference's
+block recurrence is compared too, with the bound that recurrence has against
+the exact result (see recurrence_bound)."""
 
 import argparse
 
@@ -13,6 +19,8 @@ import pytest
 import torch
 
 import bench
+from conftest import record_parity
+from jetstream_pt_amd import attention_kernel as ak
 from oracle import Env as OEnv
 from oracle import attention as oattn
 from oracle import kv_cache as okv
@@ -21,7 +29,7 @@ from oracle import quant as oquant
 from oracle.attn_layers import Int8KVAttentionKernel as OInt8Attn
 
 pytestmark = pytest.mark.gpu
-ATOL, RTOL = 1e-2, 1e-2  # attention outputs (bf16), as the reference's own kernel tests use
+ATOL, RTOL = 1e-2, 2.0 ** -8  # attention outputs (bf16): 1e-2 plus the output's own half-ulp
 
 
 def args(layers, **more):
@@ -32,10 +40,30 @@ def as_np(x):
   return x.cpu().numpy() if isinstance(x, torch.Tensor) else np.asarray(x)
 
 
-def close(got, want, rtol=RTOL):
-  got, want = got.float().cpu(), want.float()
-  bad = (got - want).abs() > ATOL + rtol * want.abs()
-  assert not bad.any(), f"{int(bad.sum())} outputs differ, worst {float((got - want).abs().max())}"
+def close(got, want, name, extra=None):
+  """|got - want| <= 1e-2 + 2^-8 |want| (+ extra, a tensor broadcastable to them)."""
+  got, want = got.double().cpu(), want.double()
+  err = record_parity(name, got, want)
+  bound = ATOL + RTOL * want.abs()
+  if extra is not None:
+    bound = bound + extra
+  bad = err > bound
+  assert not bad.any(), f"{name}: {int(bad.sum())} outputs differ, worst {float(err.max())}"
+
+
+def recurrence_bound(lengths, v_codes, v_scale, hq, block=512):
+  """How far the reference's ragged recurrence (attention_kernel.py:289-329) may
+  stray from the exact softmax attention: it keeps the running output
+  normalised and rounds it to bf16 after every block of `block` positions, a
+  relative 2^-9 of a value that is a convex combination of the dequantised
+  value rows seen so far, so at most max|v| in magnitude; later blocks only
+  scale that error down.  Bound per (slot, kv head): blocks * 2^-9 * max|scale * code|.
+  Returns it shaped (batch, hq, 1, 1) for outputs (batch, hq, 1, dim)."""
+  b, hkv = v_codes.shape[0], v_codes.shape[1]
+  vmax = (v_codes.float().abs() * v_scale.float()).amax(dim=(2, 3)).cpu()  # (b, hkv)
+  blocks = ((lengths.cpu().float() + block - 1) // block).clamp(min=1).reshape(b, 1)
+  per_head = blocks * 2.0 ** -9 * vmax
+  return per_head.repeat_interleave(hq // hkv, dim=1).reshape(b, hq, 1, 1).double().cpu()
 
 
 def test_c1_dense_bf16_eager_update_and_attention():
@@ -50,11 +78,12 @@ def test_c1_dense_bf16_eager_update_and_attention():
     want[b.to(want.device), :, pos.to(want.device), :] = new[:, :, 0, :]
     assert torch.equal(after, want)
   want, _, _ = oattn.closed_form(w["xq"].cpu(), cache.cache_k.cpu(), cache.cache_v.cpu(), mask=w["mask"].cpu())
-  close(out, want)
+  close(out, want, "c1/closed_form")
 
 
-def dense_int8_step_checks(w, batch, hkv):
+def dense_int8_step_checks(w, batch, hkv, name):
   cache, lengths = w["cache"], w["lengths"]
+  hq = w["xq"].shape[1]
   nl = cache.cache_k.shape[0]
   before = [t.clone() for t in (cache.cache_k, cache.cache_v, cache.k_scaler, cache.v_scaler)]
   out = w["step"](0)
@@ -77,19 +106,23 @@ def dense_int8_step_checks(w, batch, hkv):
   want = OInt8Attn(oenv, 0)(w["xq"].cpu(), w["xk"].cpu(), w["xv"].cpu(), None, ocache, start=None, end=lengths)
   # the reference recurrence rounds the running output to bf16 after every block of 512
   # positions, so on long slots it strays a few bf16 steps from the exact result
-  close(out, want, rtol=8 * 2.0 ** -7)
+  close(out, want, f"{name}/reference_recurrence",
+        extra=recurrence_bound(lengths, before[1][0], before[3][0], hq))
+  rms = float((out.double().cpu() - want.double()).pow(2).mean().sqrt())
+  # two results rounded to bf16 (values of magnitude around 1 to 6): their rms distance is that of
+  # the roundings, a few thousandths (observed 2.1e-3 on C3, 2.6e-3 on C2)
+  assert rms < 5e-3, f"rms distance to the recurrence restatement {rms}"
   # and slot by slot against the float64 closed form over cache ++ new token
+  # (a full slot attends all of its cache and the token)
   seq = cache.cache_k.shape[3]
   for b in range(batch):
-    n = int(lengths[b])
-    if n >= seq:
-      continue
+    n = min(int(lengths[b]), seq)
     k = torch.cat([before[0][0, b, :, :n], stash["k"][0].reshape(batch, hkv, 1, bench.D)[b]], dim=1).cpu()
     v = torch.cat([before[1][0, b, :, :n], stash["v"][0].reshape(batch, hkv, 1, bench.D)[b]], dim=1).cpu()
     ks = torch.cat([before[2][0, b, 0, :n, 0], stash["k"][1].reshape(batch)[b:b + 1]]).reshape(1, 1, n + 1, 1).cpu()
     vs = torch.cat([before[3][0, b, 0, :n, 0], stash["v"][1].reshape(batch)[b:b + 1]]).reshape(1, 1, n + 1, 1).cpu()
     exact, _, _ = oattn.closed_form(w["xq"][b:b + 1].cpu(), k[None], v[None], k_scale=ks, v_scale=vs)
-    close(out[b:b + 1], exact)
+    close(out[b:b + 1], exact, f"{name}/closed_form")
   # the remaining layers, then finalize(): every layer's row pos[b] holds its stash, nothing else moved
   stashes = [stash]
   for i in range(1, nl):
@@ -100,7 +133,9 @@ def dense_int8_step_checks(w, batch, hkv):
   torch.cuda.synchronize()
   pos = lengths.long().to(cache.cache_k.device)
   b = torch.arange(batch, device=pos.device)
-  ok = pos < cache.cache_k.shape[3]  # a full slot has no row left: nothing is written for it
+  ok = pos < cache.cache_k.shape[3]  # a full slot has no row left: nothing is written for it ...
+  bits = ak.check_status()           # ... and the step's plan says so (no launch gave up: it would raise)
+  assert bool(bits & ak.STATUS_SLOT_FULL) == bool((~ok).any())
   for l, st in enumerate(stashes):
     for which, (codes, scale) in (("k", st["k"]), ("v", st["v"])):
       want_c = before[0 if which == "k" else 1][l].clone()
@@ -114,11 +149,13 @@ def dense_int8_step_checks(w, batch, hkv):
 
 
 def test_c2_int8_mha_decode_step():
-  dense_int8_step_checks(bench.build_c2(torch, args(2)), 96, 32)
+  w = bench.build_c2(torch, args(2, full_slot=True))  # slot 0 at 2048 = max_cache_len: a full slot
+  assert int(w["lengths"].max()) == 2048 and int(w["lengths"].min()) >= 128
+  dense_int8_step_checks(w, 96, 32, "c2")
 
 
 def test_c3_ragged_gqa_int8_decode_step():
-  dense_int8_step_checks(bench.build_c3(torch, args(2)), 128, 8)
+  dense_int8_step_checks(bench.build_c3(torch, args(2)), 128, 8, "c3")
 
 
 def replay_manager(w, seed, total, ps, max_pages, batch):
@@ -159,6 +196,9 @@ def paged_attention_subset(w, out, layer, slots, int8):
   pam, ps = w["pam"], pk.shape[2]
   for b in slots:
     n = int(pam.lengths[b])
+    if n == 0:  # a retired slot attends nothing
+      assert not out[b].any()
+      continue
     pages = torch.from_numpy(as_np(pam.page_indices[b, : (n + ps - 1) // ps]).astype(np.int64)).to(pk.device)
     k = pk[:, pages].reshape(pk.shape[0], -1, bench.D)[:, :n].cpu()
     v = pv[:, pages].reshape(pk.shape[0], -1, bench.D)[:, :n].cpu()
@@ -168,7 +208,7 @@ def paged_attention_subset(w, out, layer, slots, int8):
       ks = sk[:, pages].reshape(1, 1, -1, 1)[:, :, :n].cpu()
       vs = sv[:, pages].reshape(1, 1, -1, 1)[:, :, :n].cpu()
     want, _, _ = oattn.closed_form(w["xq"][b:b + 1].cpu(), k[None], v[None], k_scale=ks, v_scale=vs, sm_scale=1.0)
-    close(out[b:b + 1], want)
+    close(out[b:b + 1], want, ("c5" if int8 else "c4") + "/closed_form")
 
 
 @pytest.mark.parametrize("host_alloc", [False, True])

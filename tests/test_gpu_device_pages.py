@@ -278,3 +278,68 @@ def test_paged_decode_steps_device_allocator_equals_host_allocator(int8, fused):
     same_output(out_d, want, f"replay {step}")
     compare(f"replay {step}")
   dp.check()
+
+
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("int8", [False, True])
+def test_a_decode_step_without_a_free_page_drops_the_token_and_touches_no_other_page(int8, fused):
+  """The pool runs out in a decode step (the reference raises queue.Empty before
+  anything is written, page_attention_manager.py:55-64).  On the device the
+  slots that were served get their pages as usual; a slot that was not gets page
+  id -1 in its index column and table cell, its length stays, and no page -
+  in particular none that belongs to another slot, and not the sentinel page -
+  receives its token, with a separate append launch or with the attention launch
+  appending.  check() raises queue.Empty once and clears the record."""
+  from jetstream_pt_amd import cache_manager as cm
+  from jetstream_pt_amd import layers
+  from jetstream_pt_amd.environment import JetEngineEnvironment, JetEngineEnvironmentData
+  from jetstream_pt_amd.page_attention_manager import DevicePageAttentionManager
+  g = torch.Generator().manual_seed(77 + int(int8) + 2 * int(fused))
+  b, hq, hkv, p, ps, d, mp = 4, 8, 2, 9, 32, 128, 4
+  env = JetEngineEnvironment(JetEngineEnvironmentData(batch_size=b, paged_attention_total_num_pages=p,
+                                                      paged_attention_page_size=ps))
+  dp = DevicePageAttentionManager(b, p, ps, mp, device=DEV)
+  cache = (cm.Int8PageKVCacheGenerate if int8 else cm.PageKVCacheGenerate).empty((hkv, p, ps, d), DEV, env)
+  cache.page_attention_manager = dp
+  # 2 + 2 + 2 + 1 pages taken, two left (the last of them is the sentinel id 8);
+  # slots 0, 1 and 2 all sit on a page boundary: three requests for two pages
+  lens = np.array([64, 64, 64, 5], dtype=np.int32)
+  dp.reserve_pages_insert_many(np.arange(b, dtype=np.int32), lens)
+  for t in (cache.cache_k, cache.cache_v):
+    if int8:
+      t.random_(-127, 128)
+    else:
+      t.normal_()
+  if int8:
+    cache.k_scaler.uniform_(0.01, 0.05)
+    cache.v_scaler.uniform_(0.01, 0.05)
+  dlens = torch.from_numpy(lens).to(DEV)
+  table_before = dp.page_indices.clone()
+  saved = [t.clone() for t in ((cache.cache_k, cache.cache_v) + ((cache.k_scaler, cache.v_scaler) if int8 else ()))]
+  xq = torch.randn((b, hq, 1, d), generator=g).to(torch.bfloat16).to(DEV)
+  xk = torch.randn((b, hkv, 1, d), generator=g).to(torch.bfloat16).to(DEV)
+  xv = torch.randn((b, hkv, 1, d), generator=g).to(torch.bfloat16).to(DEV)
+  kern = (layers.Int8KVAttentionKernel if int8 else layers.AttentionKernel)(env, 0, fuse_new_token=fused)
+  cache.page_token_indices = dp.decode_step(dlens)
+  assert kern._will_append_in_launch(xq, cache, cache.cache_k) == fused
+  kern(xq, xk, xv, None, cache)
+  torch.cuda.synchronize()
+  idx = cache.page_token_indices.to_host()
+  assert idx[2].tolist() == [0, 1, 2, 3]
+  assert idx[0].tolist() == [7, 8, -1, int(table_before[3, 0])]          # slots 0, 1 served in order, slot 2 not
+  assert dp.lengths.cpu().tolist() == [65, 65, 64, 6]
+  table = dp.page_indices.cpu()
+  assert table[0, 2] == 7 and table[1, 2] == 8 and table[2, 2] == -1
+  assert dp.unused_page_ids().tolist() == []
+  # pages: exactly the rows (page 7, 0), (page 8, 0) and (slot 3's page, 5) changed
+  now = (cache.cache_k, cache.cache_v) + ((cache.k_scaler, cache.v_scaler) if int8 else ())
+  written = [(7, 0), (8, 0), (int(table_before[3, 0]), 5)]
+  for before, after in zip(saved, now):
+    changed = (before != after)
+    while changed.dim() > 3:
+      changed = changed.any(dim=-1)
+    changed = changed.any(dim=0)  # (pages, rows in a page)
+    assert sorted(map(tuple, changed.nonzero().tolist())) == sorted(written)
+  with pytest.raises(queue.Empty):
+    dp.check()
+  dp.check()  # the record was cleared

@@ -121,3 +121,32 @@ def test_reference_scenario_update_finalize_dequant():
         nk, nv = nk[layer], nv[layer]
       assert torch.allclose(k.float(), nk[:, :, pos:pos + 1].float(), atol=0.1)
       assert torch.allclose(v.float(), nv[:, :, pos:pos + 1].float(), atol=0.1)
+
+
+def test_prefill_cache_pretends_to_be_quantised():
+  """cache_manager.py:42-69: KVCachePrefill keeps K/V as they are; with
+  kv_quantize it returns the 8-tuple Int8KVAttentionKernel unpacks
+  (layers.py:677-686), scalers = bf16 ones (B, 1, T, 1), nothing quantised -
+  so attention through it equals attention over the unquantised K/V."""
+  from oracle import attention as A
+  from oracle.attn_layers import AttentionKernel, Int8KVAttentionKernel
+  from oracle.kv_cache import KVCachePrefill
+  g = torch.Generator().manual_seed(11)
+  t, h, d = 12, 2, 8
+  k, v, q = rnd(g, (1, h, t, d)), rnd(g, (1, h, t, d)), rnd(g, (1, h, t, d))
+  plain = KVCachePrefill()
+  assert plain.update(k, v) == (k, v) and plain.state() == (k, v)
+  cache = KVCachePrefill(kv_quantize=True)
+  ret = cache.update(k, v, 3)
+  assert len(ret) == 8 and ret[0] is k and ret[1] is v
+  assert [ret[i] for i in (2, 3, 6, 7)] == [None] * 4
+  for ones in ret[4:6]:
+    assert ones.shape == (1, 1, t, 1) and ones.dtype == torch.bfloat16 and bool((ones == 1).all())
+  assert cache.state() == (k, v) and cache.finalize() is None
+  env = Env(batch_size=1, num_layers=1, ring_buffer=False)
+  mask = torch.full((t, t), float("-inf")).triu(1).reshape(1, 1, t, t)
+  quantised_path = Int8KVAttentionKernel(env, 0)(q, k, v, mask, KVCachePrefill(kv_quantize=True))
+  plain_path = AttentionKernel(env, 0)(q, k, v, mask, KVCachePrefill())
+  assert torch.equal(quantised_path, plain_path)  # multiplying by bf16 ones changes no bit
+  exact, _, _ = A.closed_form(q, k, v, mask=mask)
+  assert (quantised_path.double() - exact).abs().max() < 5e-2
