@@ -397,6 +397,23 @@ int32_t jpt_attn_plan(const jpt_attn_args* args, int32_t paged, void* stream);
 int32_t jpt_attn_ragged(const jpt_attn_args* args, void* stream);
 int32_t jpt_attn_dense(const jpt_attn_args* args, void* stream);
 int32_t jpt_attn_paged(const jpt_attn_args* args, void* stream);
+/* jpt_attn_ragged with the workspace inside the library: a device array of
+ * JPT_ATTN_STATIC_SCRATCH_BYTES that every GPU the library runs on holds from
+ * the moment its code is loaded there until the process ends.  No counterpart
+ * in the reference; it is for callers that cannot allocate device memory -
+ * code under HIP graph capture, tight serving loops, harnesses that forbid it.
+ * The call allocates nothing (no hipMalloc, no hipFree, no allocating
+ * library routine): it plans (unless reuse_plan), attends and merges like
+ * jpt_attn_ragged, with identical results.  args->workspace and
+ * workspace_bytes are ignored.  Shapes whose workspace
+ * (jpt_attn_workspace_bytes) exceeds the array are refused with JPT_E_BADARG.
+ * All calls on one GPU share that GPU's array, which keeps the last call's
+ * plan (so reuse_plan works across calls with the same lengths): calls that
+ * overlap in time on one GPU race, whatever their streams.
+ * jpt_attn_status(NULL, ...) reads its status word on the current device. */
+#define JPT_ATTN_STATIC_SCRATCH_BYTES (8 << 20)
+int32_t jpt_attn_ragged_static(const jpt_attn_args* args, void* stream);
+
 /* Waits for `stream`, then stores the workspace's status word into *status
  * and clears it.  Bits, sticky since the last call:
  *   JPT_ATTN_STATUS_GAVE_UP    a launch gave up (see Errors above);
@@ -408,7 +425,8 @@ int32_t jpt_attn_paged(const jpt_attn_args* args, void* stream);
  *     and overwrite the last row, cache_manager.py:154-173).
  *  Synchronises: call it where the caller synchronises anyway (the
  * reference raises from inside its jitted step; a kernel cannot).  Not to be
- * called during stream capture. */
+ * called during stream capture.  workspace NULL: the library's own workspace
+ * (jpt_attn_ragged_static) on the current device. */
 int32_t jpt_attn_status(void* workspace, void* stream, int32_t* status);
 
 /* Log-sum-exp merge of two partial attention results (layers.py:539-548):

@@ -16,6 +16,8 @@
 // bytes(v_scale)) / heads-sharing-a-scale.
 #include <math.h>
 
+#include <mutex>
+
 #include "attn_common.h"
 #include "attn_plan.h"
 
@@ -371,9 +373,70 @@ int32_t jpt_attn_plan(const jpt_attn_args* args, int32_t paged, void* stream) {
   return attn_plan_launch(*args, paged != 0, static_cast<hipStream_t>(stream));
 }
 
+// ---- jpt_attn_ragged_static: the workspace is a device array of this library ----
+// Device memory that exists from the moment the code object is loaded on a GPU
+// (zero-filled then) until the process ends: callers that must not allocate
+// need no workspace of their own.  Every GPU holds its own copy at its own
+// address.
+static __device__ __align__(256) unsigned char scratch[JPT_ATTN_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];  // the array's address on each device, once asked for
+std::mutex g_scratch_mutex;
+
+// Address of `scratch` on the current device (NULL and *st set on failure).  The
+// array's name is only a handle on the host: the address comes from the runtime,
+// once per device, with that device current.
+void* static_scratch(int32_t* st) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    *st = jpt::fail(JPT_E_HIP, "hipGetDevice: %s (device %d)", hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      *st = jpt::fail(JPT_E_HIP, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *st = JPT_OK;
+  return g_scratch_ptr[dev];
+}
+}  // namespace
+
+int32_t jpt_attn_ragged_static(const jpt_attn_args* args, void* stream) {
+  using namespace jpt;
+  JPT_REQUIRE(args != nullptr, "args is NULL");
+  JPT_REQUIRE(args->batch > 0 && args->kv_heads > 0 && args->q_heads > 0 && args->q_rows > 0 &&
+                  args->q_heads % args->kv_heads == 0, "batch, heads and q_rows must be positive");
+  const int64_t need = attn_fast_workspace_bytes(*args);
+  JPT_REQUIRE(need <= JPT_ATTN_STATIC_SCRATCH_BYTES,
+              "this shape needs a workspace of %lld bytes, the library's own holds %lld: use jpt_attn_ragged "
+              "with a workspace of the caller's", static_cast<long long>(need),
+              static_cast<long long>(JPT_ATTN_STATIC_SCRATCH_BYTES));
+  int32_t st = JPT_OK;
+  void* ptr = static_scratch(&st);
+  if (ptr == nullptr) return st;
+  jpt_attn_args a = *args;
+  a.workspace = ptr;
+  a.workspace_bytes = JPT_ATTN_STATIC_SCRATCH_BYTES;
+  return attn_entry(&a, kRagged, stream);
+}
+
 int32_t jpt_attn_status(void* workspace, void* stream, int32_t* status) {
   using namespace jpt;
-  JPT_REQUIRE(workspace != nullptr && status != nullptr, "workspace and status must not be NULL");
+  JPT_REQUIRE(status != nullptr, "status must not be NULL");
+  if (workspace == nullptr) {  // the library's own workspace on the current device
+    int32_t st = JPT_OK;
+    workspace = static_scratch(&st);
+    if (workspace == nullptr) return st;
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   int32_t word = 0;
   JPT_HIP(hipMemcpyAsync(&word, workspace, sizeof(word), hipMemcpyDeviceToHost, s));

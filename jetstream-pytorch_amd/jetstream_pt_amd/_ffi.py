@@ -25,6 +25,7 @@ OK, E_BADARG, E_NOPAGES, E_PAGE_OVERFLOW, E_HIP = 0, -1, -2, -3, -4
 BF16, F32, I8 = 0, 1, 2
 ROUND_TRUNC, ROUND_RNE = 0, 1
 ATTN_WS_STATE_BYTES = 65536
+ATTN_STATIC_SCRATCH_BYTES = 8 << 20
 MAX_LINE_TENSORS = 4
 
 _c = ctypes
@@ -137,6 +138,7 @@ _sig("jpt_attn_ragged", _i32, _c.POINTER(AttnArgs), _vp)
 _sig("jpt_attn_dense", _i32, _c.POINTER(AttnArgs), _vp)
 _sig("jpt_attn_paged", _i32, _c.POINTER(AttnArgs), _vp)
 _sig("jpt_attn_status", _i32, _vp, _vp, _i32p)
+_sig("jpt_attn_ragged_static", _i32, _c.POINTER(AttnArgs), _vp)
 _sig("jpt_lse_merge", _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _vp)
 _sig("jpt_pam_create", _i32, _i32, _i32, _i32, _i32, _i32p, _c.POINTER(_vp))
 _sig("jpt_pam_destroy", None, _vp)
@@ -165,7 +167,7 @@ EXPORTS = (
     "jpt_pam_free_count", "jpt_paged_append_dev", "jpt_dpam_init", "jpt_dpam_reserve_insert",
     "jpt_dpam_free", "jpt_dpam_decode_step", "jpt_decode_advance", "jpt_rope",
     "jpt_ragged_block_indices", "jpt_prefill_insert_layers", "jpt_prefill_insert_prompts",
-    "jpt_attn_status",
+    "jpt_attn_status", "jpt_attn_ragged_static",
 )
 
 
