@@ -162,7 +162,7 @@ def build_dense_int8(torch, nl, batch, hq, hkv, seq, lengths, name):
               config={"workload": name, "batch": batch, "q_heads": hq, "kv_heads": hkv, "head_dim": D,
                       "max_cache_len": seq, "layers_rotated": nl, "cached_tokens": total,
                       "kv": "int8 codes + fp32 per-token scales"},
-              kernel="attn_decode_kernel<int8> + attn_merge_kernel (one attention launch)")
+              kernel="attn_decode_kernel<int8> (one launch: chunks, then the merges of split slots)")
 
 
 def build_c3(torch, args):
@@ -231,7 +231,7 @@ def build_c1(torch, args):
                                   "all 1024 positions with an additive mask",
                       "batch": batch, "q_heads": heads, "kv_heads": heads, "head_dim": D,
                       "max_cache_len": seq, "layers_rotated": nl, "kv": "bf16"},
-              kernel="attn_decode_kernel<bf16, mask> + attn_merge_kernel (one attention launch)")
+              kernel="attn_decode_kernel<bf16, mask> (one launch: chunks, then the merges of split slots)")
 
 
 def build_paged(torch, args, int8):
@@ -409,7 +409,7 @@ def build_paged(torch, args, int8):
                       "page_size": ps, "total_pages": total, "max_pages_per_seq": max_pages, "layers_rotated": nl,
                       "kv": "int8 pages + fp32 scale pages" if int8 else "bf16 pages"},
               kernel=("attn_decode_kernel<int8, paged>" if int8 else "attn_decode_kernel<bf16, paged>") +
-                     " + attn_merge_kernel (one attention launch)")
+                     " (one launch: chunks, then the merges of split slots)")
 
 
 def build_c4(torch, args):

@@ -1,15 +1,21 @@
 // Ragged / dense / paged GQA decode attention for gfx950, head_dim 128: host
-// side, planning kernel and partial-merge kernel.  The streaming attention
+// side and planning kernel.  The streaming attention
 // kernel itself is in attn_decode_impl.h.
 //
 // Work decomposition (split-KV).  The planning kernel turns the per-slot
-// lengths into a list of chunks (slot, first position, count), longest first,
-// sized so the batch yields a few work items per persistent workgroup whatever
-// the length distribution.  A slot that fits one chunk is finished by the
-// attention kernel; the chunks of a longer slot park float32 partials
-// (o, max, sum) that the merge kernel folds.  The kernel boundary is the only
-// device-wide synchronisation: an in-kernel device-scope fence costs an L2
-// write-back and invalidate per workgroup on this part and serialises per XCD.
+// lengths into a list of chunks (slot, first position, count), sized so the
+// batch yields a few work items per persistent worker whatever the length
+// distribution.  A slot that fits one chunk is finished by the worker that
+// attends it.  A longer slot is cut into equal chunks, which come first in the
+// list (every worker starts with one of them, if there are that many); each
+// parks a float32 partial (o, max, sum) in memory and counts itself on the
+// slot's arrival counter.  Merge entries, one per split slot and KV head, fold
+// the partials into the slot's output; they are not dealt out: a worker's
+// producer wave, once its last tile has landed, takes merge entries from a
+// counter in memory for as long as there are any, while its consumers work off
+// the tiles still in the ring - whoever is done first does the merging.  One
+// launch: no second kernel, and no device-wide fence either; partials and
+// counters are written through to memory and read past the caches.
 //
 // Bound: HBM bandwidth.  Algorithmic bytes per (slot, KV head) are
 // len * 128 * (bytes(K) + bytes(V)) plus len * (bytes(k_scale) +
@@ -25,14 +31,17 @@ namespace jpt {
 namespace {
 
 constexpr int kChunkAlign = 128;
-constexpr float kLn2 = 0.6931471805599453f;
 
 // ---- workspace layout --------------------------------------------------------
 // [0, 64 KiB)   state block, zero before the first call; word 0 is the sticky
-//               give-up flag that jpt_attn_status reads and clears
-// then          sorted plan entries, per-slot chunk table, partials
+//               status word that jpt_attn_status reads and clears, words 2 and 3
+//               the numbers of work entries and of merge entries in the plan,
+//               words 16, 32, ... 128 the counters that hand out the merge
+//               entries (cleared by every plan, advanced by the same amounts by
+//               every launch)
+// then          plan entries, arrival counters (batch x kv_heads), partials
 struct Layout {
-  int64_t entries, slots, partials, total;
+  int64_t entries, arrivals, partials, total;
   int32_t max_entries;
 };
 
@@ -58,21 +67,26 @@ int32_t target_items() { return persistent_blocks() * 5 / 4; }
 
 Layout make_layout(int batch, int kv_heads, int rows) {
   Layout l;
-  l.max_entries = (batch + (target_items() + kv_heads - 1) / kv_heads + 1 + 7) / 8 * 8;
+  // one entry a slot, the extra chunks of split slots (at most the target's worth,
+  // and every split slot has at least one), and a merge entry for each split slot
+  const int extra = (target_items() + kv_heads - 1) / kv_heads + 1;
+  l.max_entries = (batch + 2 * extra + 7) / 8 * 8;
   auto up = [](int64_t x) { return (x + 255) / 256 * 256; };
   l.entries = JPT_ATTN_WS_STATE_BYTES;
-  l.slots = up(l.entries + static_cast<int64_t>(l.max_entries) * sizeof(PlanEntry));
-  l.partials = up(l.slots + static_cast<int64_t>(batch) * sizeof(SlotChunks));
-  l.total = up(l.partials + static_cast<int64_t>(l.max_entries) * kv_heads * rows * kPartFloats * 4);
+  l.arrivals = up(l.entries + static_cast<int64_t>(l.max_entries) * sizeof(PlanEntry));
+  l.partials = up(l.arrivals + static_cast<int64_t>(batch) * kv_heads * sizeof(int32_t));
+  l.total = up(l.partials + static_cast<int64_t>(batch + extra) * kv_heads * rows * kPartFloats * 4);
   return l;
 }
 
 // ---- planning kernel -----------------------------------------------------------
 // One workgroup.  chunk = max(128, total positions * kv_heads / target items,
-// rounded up to 128); each slot gets max(1, ceil(len / chunk)) entries
-// (an empty slot still needs one item per head to write its output);
-// entries are counting-sorted by tile count, longest first; records past the
-// last entry are marked unused.
+// rounded up to 128); a slot longer than that is cut into ceil(len / chunk)
+// equal chunks of whole tiles, any other slot is one entry (an empty slot still
+// needs one item per head to write its output).  Entries are counting-sorted:
+// chunks of split slots first, then whole slots, each by tile count, longest
+// first; after them one merge entry for every split slot; records past the last
+// entry are marked unused.  The arrival counters are cleared.
 // Exclusive prefix sum of `x` over the 256 threads of the planning workgroup;
 // *total gets the sum.
 __device__ __forceinline__ int plan_exclusive_scan(int x, int* total) {
@@ -99,16 +113,21 @@ __device__ __forceinline__ int plan_exclusive_scan(int x, int* total) {
 
 __global__ void __launch_bounds__(256)
 plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int target,
-            PlanEntry* entries, SlotChunks* slots, int max_entries, int32_t* status) {
+            PlanEntry* entries, int32_t* arrivals, int max_entries, int32_t* status) {
+  constexpr int kKeys = 2 * 257;  // tile count, plus 257 for the chunks of split slots
   __shared__ int s_len[kMaxPlanBatch];
   __shared__ int s_first[kMaxPlanBatch];
   __shared__ long long s_total;
-  __shared__ int s_chunk, s_entries;
-  __shared__ int s_hist[257];
-  __shared__ int s_base[257];
+  __shared__ int s_chunk, s_entries, s_merges;
+  __shared__ int s_hist[kKeys];
+  __shared__ int s_base[kKeys];
   const int tid = threadIdx.x;
-  if (tid == 0) s_total = 0;
-  for (int i = tid; i < 257; i += blockDim.x) s_hist[i] = 0;
+  if (tid == 0) {
+    s_total = 0;
+    s_merges = 0;
+  }
+  for (int i = tid; i < kKeys; i += blockDim.x) s_hist[i] = 0;
+  for (int i = tid; i < batch * kv_heads; i += blockDim.x) arrivals[i] = 0;
   __syncthreads();
   long long mine = 0;
   bool full = false;  // a slot with no room left for the step's token
@@ -132,6 +151,11 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
   __syncthreads();
   const int chunk = s_chunk;
   auto chunks_of = [&](int b) { return s_len[b] == 0 ? 1 : (s_len[b] + chunk - 1) / chunk; };
+  // positions of one chunk of slot b: the slot cut evenly, in whole tiles
+  auto chunk_len = [&](int b) {
+    const int nc = chunks_of(b);
+    return nc == 1 ? s_len[b] : ((s_len[b] + nc - 1) / nc + kTile - 1) / kTile * kTile;
+  };
   // a slot's first partial record: running sum of the chunk counts, 256 slots a pass
   {
     int base = 0;
@@ -145,95 +169,46 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     if (tid == 0) s_entries = base;
   }
   __syncthreads();
-  auto key_of = [&](int count) {
+  auto key_of = [&](int count, bool split) {
     const int tiles = (count + kTile - 1) / kTile;
-    return tiles > 256 ? 256 : tiles;
+    return (tiles > 256 ? 256 : tiles) + (split ? 257 : 0);
   };
   for (int b = tid; b < batch; b += blockDim.x) {
-    const int nc = chunks_of(b);
-    slots[b] = SlotChunks{nc, s_first[b]};
-    for (int c = 0; c < nc; ++c) atomicAdd(&s_hist[key_of(min(chunk, s_len[b] - c * chunk))], 1);
+    const int nc = chunks_of(b), cl = chunk_len(b);
+    for (int c = 0; c < nc; ++c) atomicAdd(&s_hist[key_of(min(cl, s_len[b] - c * cl), nc > 1)], 1);
   }
   __syncthreads();
   {
-    // where each tile count's entries start, longest first: thread t has key 256 - t
-    int total;
-    const int before = plan_exclusive_scan(s_hist[256 - tid], &total);
-    s_base[256 - tid] = before;
-    if (tid == 0) s_base[0] = total;
+    // where each key's entries start, largest key first: thread t of pass i has key kKeys - 1 - (256 i + t)
+    int base = 0;
+    for (int k0 = 0; k0 < kKeys; k0 += static_cast<int>(blockDim.x)) {
+      const int key = kKeys - 1 - (k0 + tid);
+      int total;
+      const int before = plan_exclusive_scan(key >= 0 ? s_hist[key] : 0, &total);
+      if (key >= 0) s_base[key] = base + before;
+      base += total;
+    }
   }
   __syncthreads();
   for (int b = tid; b < batch; b += blockDim.x) {
-    const int nc = chunks_of(b), first = s_first[b];
+    const int nc = chunks_of(b), cl = chunk_len(b), first = s_first[b];
     for (int c = 0; c < nc; ++c) {
-      const int count = min(chunk, s_len[b] - c * chunk);
-      const int at = atomicAdd(&s_base[key_of(count)], 1);
-      if (at < max_entries) entries[at] = PlanEntry{b, c * chunk, count, first + c, nc, s_len[b], {0, 0}};
+      const int count = min(cl, s_len[b] - c * cl);
+      const int at = atomicAdd(&s_base[key_of(count, nc > 1)], 1);
+      if (at < max_entries) entries[at] = PlanEntry{b, c * cl, count, first + c, nc, s_len[b], {0, 0}};
+    }
+    if (nc > 1) {  // the slot's merge entry, after every chunk and whole slot
+      const int at = s_entries + atomicAdd(&s_merges, 1);
+      if (at < max_entries) entries[at] = PlanEntry{b, -1, 0, first, nc, s_len[b], {0, 0}};
     }
   }
-  for (int i = s_entries + tid; i < max_entries; i += blockDim.x)
+  __syncthreads();
+  for (int i = s_entries + s_merges + tid; i < max_entries; i += blockDim.x)
     entries[i] = PlanEntry{-1, 0, 0, 0, 0, 0, {0, 0}};
-}
-
-// Folds the partials of every slot that was split into several chunks: one
-// workgroup per (slot, KV head), 16 lanes a row, eight consecutive outputs a
-// lane.  A lane loads its share of up to eight chunks - outputs, maxima and
-// sums alike - in one batch of independent loads, so a slot of up to eight
-// chunks costs one memory round trip; longer ones are folded batch by batch.
-constexpr int kMergeBatch = 8;
-__global__ void __launch_bounds__(256) attn_merge_kernel(FastParams p) {
-  const jpt_attn_args& a = p.a;
-  const int b = blockIdx.x / a.kv_heads, h = blockIdx.x % a.kv_heads;
-  const SlotChunks sc = p.slots[b];
-  const int R = p.rows, n = sc.n_chunks;
-  const int row = threadIdx.x >> 4, d0 = 8 * (threadIdx.x & 15);
-  if (n <= 1 || row >= R) return;
-  const int64_t rec = static_cast<int64_t>(R) * kPartFloats;
-  const float* base = p.partials + (static_cast<int64_t>(sc.first_part) * a.kv_heads + h) * rec + row * kPartFloats;
-  const int64_t step = static_cast<int64_t>(a.kv_heads) * rec;
-  float M = -INFINITY, L = 0.f;
-  float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int c0 = 0; c0 < n; c0 += kMergeBatch) {
-    float4 x[kMergeBatch], y[kMergeBatch];
-    float2 ml[kMergeBatch];
-#pragma unroll
-    for (int c = 0; c < kMergeBatch; ++c) {
-      ml[c] = make_float2(-INFINITY, 0.f);
-      x[c] = y[c] = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (c0 + c < n) {
-        const float* src = base + (c0 + c) * step;
-        ml[c] = *reinterpret_cast<const float2*>(src + kD);
-        x[c] = *reinterpret_cast<const float4*>(src + d0);
-        y[c] = *reinterpret_cast<const float4*>(src + d0 + 4);
-      }
-    }
-    float Mb = M;
-#pragma unroll
-    for (int c = 0; c < kMergeBatch; ++c) Mb = fmaxf(Mb, ml[c].x);
-    const float keep = M == -INFINITY ? 0.f : exp2f(M - Mb);
-    L *= keep;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] *= keep;
-#pragma unroll
-    for (int c = 0; c < kMergeBatch; ++c) {
-      const float f = ml[c].x == -INFINITY ? 0.f : exp2f(ml[c].x - Mb);
-      L += ml[c].y * f;
-      o[0] += x[c].x * f; o[1] += x[c].y * f; o[2] += x[c].z * f; o[3] += x[c].w * f;
-      o[4] += y[c].x * f; o[5] += y[c].y * f; o[6] += y[c].z * f; o[7] += y[c].w * f;
-    }
-    M = Mb;
-  }
-  const int64_t q_row = (static_cast<int64_t>(b) * a.q_heads + h * p.rep) * a.q_rows + row;
-  const float inv = L > 0.f ? 1.f / L : 0.f;
-  uint4 packed;
-  packed.x = f32_to_bf16_bits(o[0] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[1] * inv)) << 16);
-  packed.y = f32_to_bf16_bits(o[2] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[3] * inv)) << 16);
-  packed.z = f32_to_bf16_bits(o[4] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[5] * inv)) << 16);
-  packed.w = f32_to_bf16_bits(o[6] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[7] * inv)) << 16);
-  *reinterpret_cast<uint4*>(static_cast<uint16_t*>(a.out) + q_row * kD + d0) = packed;
-  if (d0 == 0) {
-    if (a.out_max) a.out_max[q_row] = M * kLn2;
-    if (a.out_denom) a.out_denom[q_row] = L;
+  if (tid < kHandOutCounters) status[kStateHandOut + tid * kStateHandOutStride] = 0;
+  if (tid == 0) {
+    status[kStateEntries] = min(s_entries, max_entries);
+    status[kStateMerges] = max(min(s_entries + s_merges, max_entries) - s_entries, 0);
   }
 }
 
@@ -280,7 +255,7 @@ int32_t attn_plan_launch(const jpt_attn_args& a, bool paged, hipStream_t stream)
   JPT_REQUIRE(cap > 0, "sequence capacity must be positive");
   hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(256), 0, stream, a.lengths, a.batch, cap,
                      a.kv_heads, target_items(), reinterpret_cast<PlanEntry*>(ws + l.entries),
-                     reinterpret_cast<SlotChunks*>(ws + l.slots), l.max_entries,
+                     reinterpret_cast<int32_t*>(ws + l.arrivals), l.max_entries,
                      reinterpret_cast<int32_t*>(ws));
   return launch_status("plan_kernel");
 }
@@ -297,7 +272,7 @@ int32_t attn_fast_launch(const jpt_attn_args& a, AttnMode mode, hipStream_t stre
   FastParams p{};
   p.a = a;
   p.entries = reinterpret_cast<const PlanEntry*>(ws + l.entries);
-  p.slots = reinterpret_cast<const SlotChunks*>(ws + l.slots);
+  p.arrivals = reinterpret_cast<int32_t*>(ws + l.arrivals);
   p.partials = reinterpret_cast<float*>(ws + l.partials);
   p.rows = rows;
   p.rep = rep;
@@ -311,12 +286,7 @@ int32_t attn_fast_launch(const jpt_attn_args& a, AttnMode mode, hipStream_t stre
   if (blocks > p.total_items) blocks = p.total_items;  // total_items is a multiple of 8
   if (a.kv_dtype == JPT_I8) decode::launch_decode_i8(p, mode == kPaged, blocks, stream);
   else decode::launch_decode_bf16(p, mode == kPaged, blocks, stream);
-  int32_t st = launch_status("attn_decode_kernel");
-  if (st != JPT_OK) return st;
-  // 16 lanes a row: only as many waves as the rows need
-  const unsigned merge_threads = static_cast<unsigned>((rows * 16 + 63) / 64 * 64);
-  hipLaunchKernelGGL(attn_merge_kernel, dim3(a.batch * a.kv_heads), dim3(merge_threads), 0, stream, p);
-  return launch_status("attn_merge_kernel");
+  return launch_status("attn_decode_kernel");
 }
 
 }  // namespace jpt

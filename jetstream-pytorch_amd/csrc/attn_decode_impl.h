@@ -31,7 +31,9 @@
 // Waves never meet at a workgroup barrier after set-up: ring slots are handed
 // over through LDS counters, and the consumer that delivers the last part of an
 // item folds the parts and writes the slot's output (one chunk) or parks the
-// chunk's float32 partial (several; a second kernel folds those).  Every wait
+// chunk's float32 partial in memory and counts the chunk as arrived (several
+// chunks; a merge item at the end of some worker's sequence folds those, see
+// merge_item).  Every wait
 // is bounded: a wave that waits too long raises an abort flag, every wave of
 // the workgroup leaves, and a sticky word in the workspace's state block tells
 // the host that the launch's results are not to be used (jpt_attn_status), so
@@ -171,6 +173,35 @@ __device__ __forceinline__ float rows_max(float r) {
   return fmaxf(fmaxf(a, b), fmaxf(c, d));
 }
 
+// Combines a value over the four 16-lane rows of the wave (lanes r, 16 + r,
+// 32 + r, 48 + r end up with the same result) with the row-swap instructions
+// of gfx950: v_permlane16_swap exchanges rows 1 and 3 of one operand with rows
+// 0 and 2 of the other, v_permlane32_swap the upper half of one with the lower
+// half of the other, so two swaps and two combines do it in the vector ALU,
+// with no trip through the LDS crossbar.  The second operand is a copy the
+// optimiser cannot see through (the swap of a register with itself is not
+// what the instruction does).
+template <typename F>
+__device__ __forceinline__ float across_rows(float v, F combine) {
+  int a = __builtin_bit_cast(int, v), c = a;
+  asm volatile("" : "+v"(c));
+  const auto s16 = __builtin_amdgcn_permlane16_swap(a, c, false, false);
+  const int lo16 = s16[0], hi16 = s16[1];  // named: a bit cast straight from the element reads element 0 twice
+  v = combine(__builtin_bit_cast(float, lo16), __builtin_bit_cast(float, hi16));
+  a = __builtin_bit_cast(int, v);
+  c = a;
+  asm volatile("" : "+v"(c));
+  const auto s32 = __builtin_amdgcn_permlane32_swap(a, c, false, false);
+  const int lo32 = s32[0], hi32 = s32[1];
+  return combine(__builtin_bit_cast(float, lo32), __builtin_bit_cast(float, hi32));
+}
+__device__ __forceinline__ float max_across_rows(float v) {
+  return across_rows(v, [](float x, float y) { return fmaxf(x, y); });
+}
+__device__ __forceinline__ float sum_across_rows(float v) {
+  return across_rows(v, [](float x, float y) { return x + y; });
+}
+
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding)
 constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
 
@@ -303,6 +334,8 @@ struct Item {
   int slot, start, count, part, n_chunks, h;
   int len;  // positions of the whole slot
   bool valid;
+  // folds the partials of a split slot (part = its first partial record) instead of attending positions
+  __device__ __forceinline__ bool merge() const { return start < 0; }
 };
 
 template <typename KV, bool PAGED, int SCALE, bool MASK, int RC>
@@ -338,6 +371,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
     (&sm_folded_all[0][0])[tid] = 0;
   }
   if (tid < kGroups * C::kQBufs) (&sm_qtaken_all[0][0])[tid] = 0;
+
   if (tid == 0) sm_abort = 0;
 
   const int R = p.rows;
@@ -345,7 +379,10 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
   // are equal mod 8 when the grid is a multiple of 8.
   const int G = kGroups * static_cast<int>(gridDim.x);
   const int worker = static_cast<int>(blockIdx.x) + group * static_cast<int>(gridDim.x);
-  const int n_rounds = (p.total_items + G - 1) / G;
+  // work entries of the plan (its merge entries follow them; see the producer)
+  const int n_entries = load_uniform(p.status + kStateEntries);
+  const int n_ids = (n_entries + 7) / 8 * 8 * a.kv_heads;  // item ids that may name a work entry
+  const int n_rounds = (n_ids + G - 1) / G;
   const bool has_new = a.new_k != nullptr;
   // the new token arrives unquantised: the consumer of its tile quantises it
   const bool quant_new = std::is_same<KV, int8_t>::value && a.new_k_raw != nullptr;
@@ -367,7 +404,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
     const int m = i >> 3;
     *entry = (m / a.kv_heads) * 8 + (i & 7);
     *h = m % a.kv_heads;
-    return k < n_rounds && i < p.total_items;
+    return k < n_rounds && i < n_ids && *entry < n_entries;
   };
   // The first kListedItems rounds are read here, all at once, into LDS (one
   // memory latency for the lot, and none inside the stream); later rounds, which
@@ -449,6 +486,87 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
       }
       __builtin_amdgcn_s_sleep(1);
     }
+    return true;
+  };
+
+  // One float written through to memory / read from memory past every cache
+  // level: what workgroups on different XCDs, each behind an L2 of its own,
+  // exchange without a device-wide fence.
+  auto put = [](float* at, float x) { __hip_atomic_store(at, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM); };
+  auto get = [](const float* at) { return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM); };
+  // writes rows of outputs: 16 lanes a row, eight outputs a lane, the statistics by the row's first lane
+  auto write_row = [&](int64_t q_row, int d0, const float (&o)[8], float M, float l) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    const uint4 packed = make_uint4(pack_bf16(o[0] * inv, o[1] * inv), pack_bf16(o[2] * inv, o[3] * inv),
+                                    pack_bf16(o[4] * inv, o[5] * inv), pack_bf16(o[6] * inv, o[7] * inv));
+    *reinterpret_cast<uint4*>(static_cast<uint16_t*>(a.out) + q_row * kD + d0) = packed;
+    if (d0 == 0) {
+      if (a.out_max) a.out_max[q_row] = M * kLn2;
+      if (a.out_denom) a.out_denom[q_row] = l;
+    }
+  };
+  // A merge item: every chunk of the slot has parked its partial and been
+  // counted (merge entries come last in the plan and the chunks first, so the
+  // wait is normally over before it starts; it is bounded like every other);
+  // folds the partials and writes the slot's output.  One wave's work.
+  auto merge_item = [&](const Item& it) -> bool {
+    int32_t* counter = p.arrivals + static_cast<int64_t>(it.slot) * a.kv_heads + it.h;
+    for (int spins = 0;; ++spins) {
+      int seen = 0;
+      if (lane == 0) seen = __hip_atomic_fetch_add(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (__builtin_amdgcn_readfirstlane(seen) >= it.n_chunks) break;
+      if (spins > (kSpinLimit >> 6) || __hip_atomic_load(&sm_abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) {
+        give_up();
+        return false;
+      }
+      __builtin_amdgcn_s_sleep(32);
+    }
+    const int64_t rec = static_cast<int64_t>(R) * kPartFloats;
+    const int64_t step = static_cast<int64_t>(a.kv_heads) * rec;
+    const int64_t q_row0 = (static_cast<int64_t>(it.slot) * a.q_heads + it.h * p.rep) * a.q_rows;
+    const int d0 = 8 * (lane & 15);
+    constexpr int kBatch = 4;  // chunks loaded together
+    for (int row = lane >> 4; row < R; row += 4) {
+      const float* src = p.partials + (static_cast<int64_t>(it.part) * a.kv_heads + it.h) * rec + row * kPartFloats;
+      float M = -INFINITY, L = 0.f;
+      float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      for (int c0 = 0; c0 < it.n_chunks; c0 += kBatch) {
+        float x[kBatch][8], m[kBatch], l[kBatch];
+#pragma unroll
+        for (int c = 0; c < kBatch; ++c) {
+          m[c] = -INFINITY;
+          l[c] = 0.f;
+          if (c0 + c < it.n_chunks) {
+            const float* s = src + (c0 + c) * step;
+            m[c] = get(s + kD);
+            l[c] = get(s + kD + 1);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[c][i] = get(s + d0 + i);
+          } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[c][i] = 0.f;
+          }
+        }
+        float Mb = M;
+#pragma unroll
+        for (int c = 0; c < kBatch; ++c) Mb = fmaxf(Mb, m[c]);
+        const float keep_old = M == -INFINITY ? 0.f : fast_exp2(M - Mb);
+        L *= keep_old;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] *= keep_old;
+#pragma unroll
+        for (int c = 0; c < kBatch; ++c) {
+          const float f = m[c] == -INFINITY ? 0.f : fast_exp2(m[c] - Mb);
+          L += l[c] * f;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) o[i] += x[c][i] * f;
+        }
+        M = Mb;
+      }
+      write_row(q_row0 + row, d0, o, M, L);
+    }
+    // every chunk was counted before its partial was read: nothing touches the counter any more
+    if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return true;
   };
 
@@ -729,6 +847,37 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
       }
       __builtin_amdgcn_s_sleep(1);
     }
+    // Every tile of this worker has landed; its consumers are working off the
+    // ring.  The producer now folds split slots: it takes (merge entry, head)
+    // pairs from a counter in memory for as long as there are any - the workers
+    // that are done first do the merging, which costs the launch no tail.  The
+    // workers of workgroups equal mod 8 share one counter and the pairs equal to
+    // them mod 8 (a dozen nanoseconds per atomic add on one address: one counter
+    // for everybody would queue).  Every worker asks until it is refused once, so
+    // a launch advances a counter by exactly its pairs plus its workers, and
+    // launches that follow one another on a plan need no reset: the counter's
+    // value modulo that sum is the place in the current launch.
+    const int n_merges = load_uniform(p.status + kStateMerges);
+    const int share = worker & 7;
+    const int sharers = (G - share + 7) / 8;
+    const int pairs = n_merges * a.kv_heads;
+    const int my_pairs = pairs > share ? (pairs - share + 7) / 8 : 0;
+    const unsigned per_launch = static_cast<unsigned>(my_pairs + sharers);
+    int32_t* const hand_out = p.status + kStateHandOut + share * kStateHandOutStride;
+    for (;;) {
+      int number = 0;
+      if (lane == 0) number = __hip_atomic_fetch_add(hand_out, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned place = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(number)) % per_launch;
+      if (place >= static_cast<unsigned>(my_pairs)) break;
+      const int pair = share + 8 * static_cast<int>(place);
+      const int32_t* en = reinterpret_cast<const int32_t*>(p.entries + n_entries + pair / a.kv_heads);
+      Item it;
+      it.slot = load_uniform(en + 0); it.start = load_uniform(en + 1); it.count = 0;
+      it.part = load_uniform(en + 3); it.n_chunks = load_uniform(en + 4); it.len = load_uniform(en + 5);
+      it.h = pair % a.kv_heads;
+      it.valid = true;
+      if (it.slot < 0 || !merge_item(it)) return;
+    }
     return;
   }
 
@@ -750,8 +899,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
   float l_run = 0.f;        // this lane's share of the row sum
 
   // Takes tile number `t` of the group's stream out of the ring and
-  // accumulates it; `valid` positions of the tile count (all of them when
-  // `full_tag` says so).
+  // accumulates it; `valid` positions of the tile count.
   int cur_slot = 0, cur_h = 0;  // of the item being consumed
   // Quantising the new token of slot cur_slot, whose kv_heads bf16 rows lie one
   // after another in `area` (the tile's key or value area): arithmetic and
@@ -841,14 +989,29 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
   uint32_t keep_k = 0, keep_v = 0;
   float keep_ks = 0.f, keep_vs = 0.f;
   bool keep = false;
-  auto consume_tile = [&](int t, int valid, bool is_new, auto full_tag) -> bool {
-    constexpr bool FULL = decltype(full_tag)::value;
+  // Chunks of split slots.  A chunk's partial must be in memory, where the
+  // workgroups of every XCD see it, before the chunk is counted as arrived; the
+  // wave that parked it does not wait for that: it sends the count after its
+  // next tile (or when it is done), when its stores have long been
+  // acknowledged.
+  int32_t* owed_arrival = nullptr;  // counter of a chunk this wave parked and has not counted yet
+  auto count_parked_chunk = [&]() {
+    if (owed_arrival == nullptr) return;
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // the partial's write-through stores are acknowledged
+    if (lane == 0) __hip_atomic_fetch_add(owed_arrival, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    owed_arrival = nullptr;
+  };
+  auto consume_tile = [&](int t, int valid, bool is_new) -> bool {
+    // One body for every tile: what only the new token's tile or a chunk's last,
+    // partly filled tile need sits behind wave-uniform branches, so that the
+    // accumulators live in the same registers whichever way a tile goes.
+    const bool partial = valid != kTile;
     const int s = t % C::kSlots;
     if (!wait_for(&sm_filled[s], t / C::kSlots + 1)) return false;
     char* slot = ring + s * C::kSlotBytes;
     const char* side = slot + 2 * C::kTileBytes;
     float new_ks = 0.f, new_vs = 0.f;
-    const bool quant_here = !FULL && is_new && quant_new;
+    const bool quant_here = is_new && quant_new;
     if (quant_here) {
       const float* rope = a.new_k_rope ? a.new_k_rope + static_cast<int64_t>(cur_slot) * kD : nullptr;
       float k0, k1, v0, v1;
@@ -908,7 +1071,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
         for (int i = 0; i < 8; ++i) mk[i] = 0.f;
       }
     }
-    if (!FULL && is_new && to_pages) {  // row 0 of the tile: piece p sits at piece slot p
+    if (is_new && to_pages) {  // row 0 of the tile: piece p sits at piece slot p
       if (kLaneBytes == 2) {
         keep_k = *reinterpret_cast<const uint16_t*>(slot + lane * 2);
         keep_v = *reinterpret_cast<const uint16_t*>(slot + C::kTileBytes + lane * 2);
@@ -939,12 +1102,15 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
     for (int i = 0; i < 8; ++i) {
       float x = (i < 4 ? sa[i] : sb[i - 4]) * (SCALE ? ks[i] * c2_row : c2_row);
       if (MASK) x += mk[i] * kLog2e;
-      if (!FULL) x = pos[i] < valid ? x : -INFINITY;
       sc[i] = x;
-      tmax = fmaxf(tmax, x);
     }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+    if (partial) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sc[i] = pos[i] < valid ? sc[i] : -INFINITY;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) tmax = fmaxf(tmax, sc[i]);
+    tmax = max_across_rows(tmax);
     const float m_new = fmaxf(m_run, tmax);
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
     const float alpha = fast_exp2(m_run - m_use);
@@ -953,8 +1119,11 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
     for (int i = 0; i < 8; ++i) {
       const float pr = fast_exp2(sc[i] - m_use);
       psum += pr;
-      // a position that does not count has weight 0 whatever its scale holds
-      w[i] = SCALE ? ((FULL || pos[i] < valid) ? pr * vs[i] : 0.f) : pr;
+      w[i] = SCALE ? pr * vs[i] : pr;
+    }
+    if (SCALE && partial) {  // a position that does not count has weight 0 whatever its scale holds
+#pragma unroll
+      for (int i = 0; i < 8; ++i) w[i] = pos[i] < valid ? w[i] : 0.f;
     }
     l_run = l_run * alpha + psum;
     m_run = m_new;
@@ -968,6 +1137,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = T::mfma(tile.v_op(j), pop, acc[j]);
     if (T::kBias != 0.f) accw = T::mfma(T::ones(), pop, accw);
+    count_parked_chunk();
     return true;
   };
 
@@ -975,11 +1145,11 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
   // consumer to arrive folds the parts and writes the slot's output (one
   // chunk) or parks the chunk's partial (several).
   auto finish_item = [&](const Item& it, int seq) -> bool {
+    count_parked_chunk();
     const int buf = seq % C::kFoldBufs;
     // the buffer's previous item must have been folded out of it
     if (!wait_for(&sm_folded[buf], seq / C::kFoldBufs)) return false;
-    float l_row = l_run + __shfl_xor(l_run, 16);
-    l_row += __shfl_xor(l_row, 32);
+    const float l_row = sum_across_rows(l_run);
     if (r < R) {
       const float bias = T::kBias * accw[0];  // every element of accw is the row's weight sum
 #pragma unroll
@@ -1018,24 +1188,18 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
         o[4] += y.x * f; o[5] += y.y * f; o[6] += y.z * f; o[7] += y.w * f;
       }
       if (it.n_chunks == 1) {
-        const float inv = l > 0.f ? 1.f / l : 0.f;
-        const uint4 packed = make_uint4(pack_bf16(o[0] * inv, o[1] * inv), pack_bf16(o[2] * inv, o[3] * inv),
-                                        pack_bf16(o[4] * inv, o[5] * inv), pack_bf16(o[6] * inv, o[7] * inv));
-        *reinterpret_cast<uint4*>(static_cast<uint16_t*>(a.out) + (q_row0 + row) * kD + d0) = packed;
+        write_row(q_row0 + row, d0, o, M, l);
+      } else {  // park the chunk's partial where the workgroups of every XCD see it
+        float* dst = part + row * kPartFloats;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) put(dst + d0 + i, o[i]);
         if (d0 == 0) {
-          if (a.out_max) a.out_max[q_row0 + row] = M * kLn2;
-          if (a.out_denom) a.out_denom[q_row0 + row] = l;
-        }
-      } else {
-        float4* dst = reinterpret_cast<float4*>(part + row * kPartFloats + d0);
-        dst[0] = make_float4(o[0], o[1], o[2], o[3]);
-        dst[1] = make_float4(o[4], o[5], o[6], o[7]);
-        if (d0 == 0) {
-          part[row * kPartFloats + kD] = M;
-          part[row * kPartFloats + kD + 1] = l;
+          put(dst + kD, M);
+          put(dst + kD + 1, l);
         }
       }
     }
+    if (it.n_chunks > 1) owed_arrival = p.arrivals + static_cast<int64_t>(it.slot) * a.kv_heads + it.h;
     if (lane == 0) {
       __hip_atomic_store(&sm_arrived[buf], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       __hip_atomic_fetch_add(&sm_folded[buf], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -1087,8 +1251,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
         float amax = 0.f;
 #pragma unroll
         for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(f[i]));
-        amax = fmaxf(amax, __shfl_xor(amax, 16));
-        amax = fmaxf(amax, __shfl_xor(amax, 32));
+        amax = max_across_rows(amax);
         int e = 0;
         if (amax > 0.f && amax < INFINITY) frexpf(amax, &e);
         e = max(e, -100);
@@ -1104,8 +1267,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
         for (int kk = 0; kk < 4; ++kk)
           qop[kk] = as_op<Op>(pack_f16(f[8 * kk], f[8 * kk + 1]), pack_f16(f[8 * kk + 2], f[8 * kk + 3]),
                               pack_f16(f[8 * kk + 4], f[8 * kk + 5]), pack_f16(f[8 * kk + 6], f[8 * kk + 7]));
-        qs += __shfl_xor(qs, 16);
-        qs += __shfl_xor(qs, 32);
+        qs = sum_across_rows(qs);
         const float ncq = -T::kBias * qs;
         s_init = f32x4{ncq, ncq, ncq, ncq};
       }
@@ -1131,11 +1293,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
       if (wide_new && ti == 1 && nt - n_cache == 2) continue;  // read by the consumer of tile 0
       const bool is_new = ti < nt - n_cache;  // the new token comes first
       const int valid = is_new ? 1 : min(kTile, cur.count - (ti - (nt - n_cache)) * kTile);
-      if (valid == kTile) {
-        if (!consume_tile(base + ti, valid, false, std::true_type{})) return;
-      } else {
-        if (!consume_tile(base + ti, valid, is_new, std::false_type{})) return;
-      }
+      if (!consume_tile(base + ti, valid, is_new)) return;
     }
     if (keep) {  // this consumer had the new token's tile
       keep = false;
@@ -1162,6 +1320,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
     if (!finish_item(cur, seq++)) return;
     base += nt;
   }
+  count_parked_chunk();
 }
 
 // `workers` groups are wanted; a workgroup holds kGroups of them.

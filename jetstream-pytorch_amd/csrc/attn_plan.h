@@ -1,5 +1,5 @@
-// Plan records and kernel parameters shared by the planning kernel, the
-// streaming attention kernel and the partial-merge kernel.
+// Plan records and kernel parameters shared by the planning kernel and the
+// streaming attention kernel.
 #pragma once
 
 #include "common.h"
@@ -13,26 +13,33 @@ constexpr int kPartFloats = kD + 4;  // a partial's row: o[128], max, sum, 2 unu
 
 struct PlanEntry {
   int32_t slot;        // -1: unused record
-  int32_t start;       // first position of the chunk
-  int32_t count;       // positions in the chunk (0 for an empty slot)
-  int32_t part;        // index of this chunk's partial record
+  int32_t start;       // first position of the chunk; -1: a merge entry (see `part`)
+  int32_t count;       // positions in the chunk (0 for an empty slot or a merge entry)
+  int32_t part;        // index of this chunk's partial record; merge entry: of the slot's first one
   int32_t n_chunks;    // chunks of this slot
   int32_t slot_len;    // positions of the whole slot
   int32_t pad[2];
 };
-struct SlotChunks {
-  int32_t n_chunks, first_part;
-};
+
+// words of the workspace's state block
+constexpr int kStateStatus = 0;    // sticky JPT_ATTN_STATUS_* bits
+constexpr int kStateEntries = 2;   // plan entries that are work items (chunks and whole slots)
+constexpr int kStateMerges = 3;    // merge entries, which follow them
+// merge entries handed out, one counter for the workers of workgroups equal mod 8
+// (one XCD), each in a cache line of its own (see the streaming kernel)
+constexpr int kStateHandOut = 16;
+constexpr int kStateHandOutStride = 16;
+constexpr int kHandOutCounters = 8;
 
 struct FastParams {
   jpt_attn_args a;
   const PlanEntry* entries;
-  const SlotChunks* slots;
   float* partials;
+  int32_t* arrivals;    // per (slot, KV head): chunks of a split slot whose partial is in memory; zero between launches
   int32_t rows;         // rep * q_rows
   int32_t rep;
   int32_t total_items;  // max_entries * kv_heads
-  int32_t* status;      // word 0 of the workspace's state block: sticky, set when a wave gave up
+  int32_t* status;      // the workspace's state block (kState* words)
 };
 
 namespace decode {
