@@ -134,6 +134,16 @@ __device__ __forceinline__ void lds_poke(int* p, int v) {
   asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(v) : "memory");
 }
 
+__device__ __forceinline__ void lds_poke4(void* p, i32x4 v) {
+  const uint32_t addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_int_ptr)p));
+  asm volatile("ds_write_b128 %0, %1" : : "v"(addr), "v"(v) : "memory");
+}
+typedef __attribute__((ext_vector_type(2))) int i32x2;
+__device__ __forceinline__ void lds_poke2(void* p, i32x2 v) {
+  const uint32_t addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_int_ptr)p));
+  asm volatile("ds_write_b64 %0, %1" : : "v"(addr), "v"(v) : "memory");
+}
+
 // An LDS word every lane reads alike, as a wave-uniform (scalar) value: what
 // the producer branches on stays out of the vector condition path.
 __device__ __forceinline__ int lds_peek_uniform(const int* p) {
@@ -162,6 +172,13 @@ __device__ __forceinline__ float row_max(float v) {
   v = fmaxf(v, dpp_move<0x4E>(v));   // quad_perm [2, 3, 0, 1]
   v = fmaxf(v, dpp_move<0x141>(v));  // row_half_mirror
   v = fmaxf(v, dpp_move<0x140>(v));  // row_mirror
+  return v;
+}
+__device__ __forceinline__ float row_sum(float v) {  // over the 16 lanes of a row, in every lane of it
+  v += dpp_move<0xB1>(v);
+  v += dpp_move<0x4E>(v);
+  v += dpp_move<0x141>(v);
+  v += dpp_move<0x140>(v);
   return v;
 }
 __device__ __forceinline__ float rows_max(float r) {
@@ -342,9 +359,23 @@ template <typename KV, bool PAGED, int SCALE, bool MASK, int RC>
 __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(FastParams p) {
   using C = Config<KV, SCALE, MASK, RC>;
   const jpt_attn_args& a = p.a;
+  // The kernel's arguments span several cache lines, which the compiler would
+  // fetch one after another as the code first needs them, a trip to memory
+  // each.  One word of every line is asked for here, all at once.
+  {
+    typedef const __attribute__((address_space(4))) int* const_int_ptr;
+    const_int_ptr args = (const_int_ptr)__builtin_amdgcn_kernarg_segment_ptr();
+    int touched = 0;
+#pragma unroll
+    for (unsigned at = 0; at < sizeof(FastParams); at += 64) touched += args[at / 4];
+    asm volatile("" : : "s"(touched));
+  }
   __shared__ __attribute__((aligned(1024))) char ring_all[kGroups][C::kSlots * C::kSlotBytes];
   __shared__ __attribute__((aligned(16))) float sm_o_all[kGroups][C::kFoldBufs][kConsumers][RC][kOStride];
   __shared__ __attribute__((aligned(16))) uint16_t sm_q_all[kGroups][C::kQBufs][RC][kD];
+  // per query row, written by the producer with the row's float16 operand (int8 codes only):
+  // the power of two taken out of the row, and minus the bias term of its scores
+  __shared__ __attribute__((aligned(8))) float sm_qmeta_all[kGroups][C::kQBufs][RC][2];
   __shared__ float sm_m_all[kGroups][C::kFoldBufs][kConsumers][RC];
   __shared__ float sm_l_all[kGroups][C::kFoldBufs][kConsumers][RC];
   __shared__ int sm_filled_all[kGroups][C::kSlots];   // times the producer filled this slot
@@ -359,9 +390,16 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int hw_wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, and known to be
-  const int group = hw_wave / kGroupWaves;
+  // Waves of a workgroup go round the four SIMDs in order.  Waves 0 and 1 are
+  // the producers, which mostly sleep; waves 4 and 5, on the same SIMDs, are
+  // each group's consumer 0, which has its SIMD nearly to itself; consumers 1
+  // and 2 of both groups share SIMDs 2 and 3 in pairs.  (With both producers
+  // on one SIMD and the six consumers on the other three, long slots ran 5 %
+  // slower.)
+  static_assert(kGroups == 2 && kConsumers == 3, "the role table below is for two groups of 1 + 3 waves");
+  const int group = static_cast<int>((0xE2u >> hw_wave) & 1u);                  // 0 1 0 0 0 1 1 1
   // role index: consumers 0..kConsumers-1, producer kConsumers
-  const int wave = hw_wave % kGroupWaves == 0 ? kConsumers : hw_wave % kGroupWaves - 1;
+  const int wave = static_cast<int>((0x909Fu >> (2 * hw_wave)) & 3u);           // 3 3 1 2 0 0 1 2
   for (int i = tid; i < kGroups * C::kSlots; i += kThreads) {
     (&sm_filled_all[0][0])[i] = 0;
     (&sm_freed_all[0][0])[i] = 0;
@@ -379,8 +417,20 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
   // are equal mod 8 when the grid is a multiple of 8.
   const int G = kGroups * static_cast<int>(gridDim.x);
   const int worker = static_cast<int>(blockIdx.x) + group * static_cast<int>(gridDim.x);
-  // work entries of the plan (its merge entries follow them; see the producer)
+  // Work entries of the plan (its merge entries follow them; see the producer).
+  // The producer wave asks for its first kListedItems records before anything
+  // looks at this count (the index is kept inside the entry array): count and
+  // records are in flight together, one memory latency for both.
   const int n_entries = load_uniform(p.status + kStateEntries);
+  int4 listed0 = make_int4(-1, 0, 0, 0), listed1 = make_int4(0, 0, 0, 0);
+  if (wave == kConsumers) {
+    const int j = (lane & 1) ? (G - 1 - worker) : worker;
+    const int i = lane * G + j;
+    const int entry = ((i >> 3) / a.kv_heads) * 8 + (i & 7);
+    const int4* en = reinterpret_cast<const int4*>(p.entries + min(entry, p.total_items / a.kv_heads - 1));
+    listed0 = en[0];
+    listed1 = en[1];
+  }
   const int n_ids = (n_entries + 7) / 8 * 8 * a.kv_heads;  // item ids that may name a work entry
   const int n_rounds = (n_ids + G - 1) / G;
   const bool has_new = a.new_k != nullptr;
@@ -412,6 +462,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
   char* const ring = ring_all[group];
   auto& sm_o = sm_o_all[group];
   auto& sm_q = sm_q_all[group];
+  auto& sm_qmeta = sm_qmeta_all[group];
   auto& sm_m = sm_m_all[group];
   auto& sm_l = sm_l_all[group];
   int* const sm_filled = sm_filled_all[group];
@@ -423,16 +474,10 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
   int (*const sm_pages)[kStagedPages] = sm_pages_all[PAGED ? group : 0];
   if (wave == kConsumers) {
     int entry, h;
-    const bool in_range = item_index(lane, &entry, &h);
-    int4 e0 = make_int4(-1, 0, 0, 0), e1 = make_int4(0, 0, 0, 0);
-    if (in_range) {
-      const int4* en = reinterpret_cast<const int4*>(p.entries + entry);
-      e0 = en[0];
-      e1 = en[1];
-    }
+    if (!item_index(lane, &entry, &h)) listed0 = make_int4(-1, 0, 0, 0);
     // slot, start, count, part | n_chunks, head, valid, slot length
-    *reinterpret_cast<int4*>(&sm_items[lane][0]) = e0;
-    *reinterpret_cast<int4*>(&sm_items[lane][4]) = make_int4(e1.x, h, e0.x >= 0 ? 1 : 0, e1.y);
+    *reinterpret_cast<int4*>(&sm_items[lane][0]) = listed0;
+    *reinterpret_cast<int4*>(&sm_items[lane][4]) = make_int4(listed1.x, h, listed0.x >= 0 ? 1 : 0, listed1.y);
   }
   __syncthreads();
   auto unpack_item = [&](int4 e0, int4 e1) -> Item {
@@ -611,6 +656,53 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
     // order, so with `out` loads still counted as outstanding (the wave's own
     // vector-memory counter, read without waiting) the first
     // loads_issued - out loads are complete.
+    // int8 codes meet the query as float16 (see Tile<int8_t>): the rows of an
+    // item, which arrive as bf16, are turned into that operand here, once, in
+    // place, before the item's first tile is handed over - by the wave with
+    // time to spare, not by each consumer.  A row is scaled by the power of two
+    // that puts its largest magnitude in [2^13, 2^14) (exact; the power goes
+    // into the scores' factor), and the bias term 1152 * sum(q) of the row is
+    // summed up.  16 lanes a row, eight elements a lane.
+    int q_converted = 0;  // items whose rows have been converted
+    auto convert_q = [&](int buf) {
+      for (int j = 0; j < q_loads; ++j) {
+        const int piece = 64 * j + lane;
+        const bool live = piece < R * 16;
+        uint16_t* at = &sm_q[buf][0][0] + (live ? piece : 0) * 8;
+        const i32x4 raw = lds_peek4(reinterpret_cast<const int*>(at));
+        float f[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          f[2 * i] = __uint_as_float(static_cast<uint32_t>(raw[i]) << 16);
+          f[2 * i + 1] = __uint_as_float(static_cast<uint32_t>(raw[i]) & 0xffff0000u);
+        }
+        float amax = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(f[i]));
+        amax = row_max(amax);
+        int e = 0;
+        if (amax > 0.f && amax < INFINITY) frexpf(amax, &e);
+        e = max(e, -100);
+        const float up = ldexpf(1.f, 14 - e);
+        float qs = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          f[i] *= up;
+          qs += f[i];
+        }
+        qs = row_sum(qs);
+        if (live) {
+          const i32x4 ops = {static_cast<int>(pack_f16(f[0], f[1])), static_cast<int>(pack_f16(f[2], f[3])),
+                             static_cast<int>(pack_f16(f[4], f[5])), static_cast<int>(pack_f16(f[6], f[7]))};
+          lds_poke4(at, ops);
+          if ((piece & 15) == 0) {
+            const i32x2 meta = {__builtin_bit_cast(int, ldexpf(1.f, e - 14)),
+                                __builtin_bit_cast(int, -Tile<KV>::kBias * qs)};
+            lds_poke2(&sm_qmeta[buf][piece >> 4][0], meta);
+          }
+        }
+      }
+    };
     auto signal_landed = [&]() {
       const uint32_t ib = __builtin_amdgcn_s_getreg(0xF807);  // HW_REG_IB_STS, all 32 bits
       const int out = static_cast<int>((ib & 0xF) | (((ib >> 22) & 0x3) << 4));
@@ -619,6 +711,12 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
         const int need = sig_base + C::kLoadsPerTile + (((carries_q >> (signalled & 63)) & 1) ? q_loads : 0) +
                          (PAGED ? static_cast<int>((carries_p >> (signalled & 63)) & 1) : 0);
         if (done < need) break;
+        if (Tile<KV>::kBias != 0.f && ((carries_q >> (signalled & 63)) & 1)) {
+          // the tile's item starts here and its query rows landed before it
+          convert_q(q_converted % C::kQBufs);
+          ++q_converted;
+        }
+        // LDS takes a wave's writes in order: the operand is there before this word
         lds_poke(&sm_filled[sig_slot], sig_round);  // every lane stores the same word
         sig_base = need;
         carries_q &= ~(1ull << (signalled & 63));
@@ -1231,45 +1329,15 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
         u[kk] = make_uint4(0, 0, 0, 0);
         if (r < R) u[kk] = *reinterpret_cast<const uint4*>(&sm_q[qb][r][32 * g + 8 * kk]);
       }
-      if (T::kBias == 0.f) {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) qop[kk] = __builtin_bit_cast(Op, u[kk]);
-      } else {
-        // float16 operand: the row is scaled by a power of two that puts its
-        // largest magnitude in [2^13, 2^14) (exact; the power goes into
-        // c2_row), and the bias term 1152 * sum(q) of the row is summed up
-        float f[32];
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          const uint32_t wds[4] = {u[kk].x, u[kk].y, u[kk].z, u[kk].w};
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            f[8 * kk + 2 * i] = __uint_as_float(wds[i] << 16);
-            f[8 * kk + 2 * i + 1] = __uint_as_float(wds[i] & 0xffff0000u);
-          }
-        }
-        float amax = 0.f;
-#pragma unroll
-        for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(f[i]));
-        amax = max_across_rows(amax);
-        int e = 0;
-        if (amax > 0.f && amax < INFINITY) frexpf(amax, &e);
-        e = max(e, -100);
-        const float up = ldexpf(1.f, 14 - e);
-        c2_row = c2 * ldexpf(1.f, e - 14);
-        float qs = 0.f;
-#pragma unroll
-        for (int i = 0; i < 32; ++i) {
-          f[i] *= up;
-          qs += f[i];
-        }
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk)
-          qop[kk] = as_op<Op>(pack_f16(f[8 * kk], f[8 * kk + 1]), pack_f16(f[8 * kk + 2], f[8 * kk + 3]),
-                              pack_f16(f[8 * kk + 4], f[8 * kk + 5]), pack_f16(f[8 * kk + 6], f[8 * kk + 7]));
-        qs = sum_across_rows(qs);
-        const float ncq = -T::kBias * qs;
-        s_init = f32x4{ncq, ncq, ncq, ncq};
+      for (int kk = 0; kk < 4; ++kk) qop[kk] = __builtin_bit_cast(Op, u[kk]);
+      if (T::kBias != 0.f) {
+        // float16 operand made by the producer, with the row's power of two and
+        // the bias term of its scores beside it
+        float2 meta = make_float2(1.f, 0.f);
+        if (r < R) meta = *reinterpret_cast<const float2*>(&sm_qmeta[qb][r][0]);
+        c2_row = c2 * meta.x;
+        s_init = f32x4{meta.y, meta.y, meta.y, meta.y};
       }
       // taken (the release waits for the reads above)
       if (lane == 0)
