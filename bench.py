@@ -488,6 +488,23 @@ def run_traffic_probe(args):
   from jetstream_pt_amd import attention_kernel as ak
 
   torch.cuda.set_device(0)
+  if args.workload != "c3":
+    # the workload's own attention launch (c4: bf16 pages), eight times, each next to a calibration copy
+    w = WORKLOADS[args.workload](torch, args)
+    if "before_pass" in w:
+      w["before_pass"]()
+    w["step"](0)  # the step's page allocation and plan
+    src = torch.empty(PROBE_COPY_BYTES // 4, dtype=torch.float32, device=DEV).normal_()
+    dst = torch.empty_like(src)
+    for i in range(8):
+      w["attn_only"](i)
+      dst.copy_(src)
+    torch.cuda.synchronize()
+    launch_bytes = w["bytes_now"]()[1] if "bytes_now" in w else w["attn_bytes"]
+    print(json.dumps({"probe": "traffic", "workload": args.workload, "attention_launches": 8, "copies": 8,
+                      "copy_bytes_read": PROBE_COPY_BYTES, "copy_bytes_written": PROBE_COPY_BYTES,
+                      "attn_algorithmic_bytes": int(launch_bytes)}))
+    return
   nl = 4
   lengths = seeded_lengths(torch).to(DEV)
   k = torch.empty((nl, B, HKV, S, D), dtype=torch.int8, device=DEV)

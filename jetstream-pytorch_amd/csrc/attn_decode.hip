@@ -6,16 +6,19 @@
 // lengths into a list of chunks (slot, first position, count), sized so the
 // batch yields a few work items per persistent worker whatever the length
 // distribution.  A slot that fits one chunk is finished by the worker that
-// attends it.  A longer slot is cut into equal chunks, which come first in the
-// list (every worker starts with one of them, if there are that many); each
-// parks a float32 partial (o, max, sum) in memory and counts itself on the
-// slot's arrival counter.  Merge entries, one per split slot and KV head, fold
-// the partials into the slot's output; they are not dealt out: a worker's
-// producer wave, once its last tile has landed, takes merge entries from a
-// counter in memory for as long as there are any, while its consumers work off
-// the tiles still in the ring - whoever is done first does the merging.  One
-// launch: no second kernel, and no device-wide fence either; partials and
-// counters are written through to memory and read past the caches.
+// attends it.  A longer slot is cut into equal chunks.  Cut in two, its chunks
+// go to the two groups of waves of one workgroup, which fold them through LDS:
+// nothing of such a slot touches memory but its output.  Cut in three or more,
+// its chunks come first in the list (every worker starts with one of them, if
+// there are that many); each parks a float32 partial (o, max, sum) in memory
+// and counts itself on the slot's arrival counter.  Merge entries, one per such
+// slot and KV head, fold the partials into the slot's output; they are not
+// dealt out: a worker's producer wave, once its last tile has landed, takes
+// merge entries from a counter in memory for as long as there are any, while
+// its consumers work off the tiles still in the ring - whoever is done first
+// does the merging.  One launch: no second kernel, and no device-wide fence
+// either; partials and counters are written through to memory and read past
+// the caches.
 //
 // Bound: HBM bandwidth.  Algorithmic bytes per (slot, KV head) are
 // len * 128 * (bytes(K) + bytes(V)) plus len * (bytes(k_scale) +
@@ -70,7 +73,8 @@ Layout make_layout(int batch, int kv_heads, int rows) {
   // one entry a slot, the extra chunks of split slots (at most the target's worth,
   // and every split slot has at least one), and a merge entry for each split slot
   const int extra = (target_items() + kv_heads - 1) / kv_heads + 1;
-  l.max_entries = (batch + 2 * extra + 7) / 8 * 8;
+  // ... and the places a half-filled round of paired chunks leaves empty
+  l.max_entries = (batch + 2 * extra + persistent_blocks() / kv_heads + 8 + 7) / 8 * 8;
   auto up = [](int64_t x) { return (x + 255) / 256 * 256; };
   l.entries = JPT_ATTN_WS_STATE_BYTES;
   l.arrivals = up(l.entries + static_cast<int64_t>(l.max_entries) * sizeof(PlanEntry));
@@ -83,10 +87,12 @@ Layout make_layout(int batch, int kv_heads, int rows) {
 // One workgroup.  chunk = max(128, total positions * kv_heads / target items,
 // rounded up to 128); a slot longer than that is cut into ceil(len / chunk)
 // equal chunks of whole tiles, any other slot is one entry (an empty slot still
-// needs one item per head to write its output).  Entries are counting-sorted:
-// chunks of split slots first, then whole slots, each by tile count, longest
-// first; after them one merge entry for every split slot; records past the last
-// entry are marked unused.  The arrival counters are cleared.
+// needs one item per head to write its output).  Entries are counting-sorted by
+// tile count, longest first: the slots cut in two (their two chunks on a pair
+// of places that one workgroup's groups walk in the same round, see below),
+// then the chunks of the other cut slots, then whole slots; after the last
+// place one merge entry for every slot cut in three or more; places nobody was
+// put on are marked unused.  The arrival counters are cleared.
 // Exclusive prefix sum of `x` over the 256 threads of the planning workgroup;
 // *total gets the sum.
 __device__ __forceinline__ int plan_exclusive_scan(int x, int* total) {
@@ -112,22 +118,24 @@ __device__ __forceinline__ int plan_exclusive_scan(int x, int* total) {
 }
 
 __global__ void __launch_bounds__(256)
-plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int target,
+plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int target, int workers,
             PlanEntry* entries, int32_t* arrivals, int max_entries, int32_t* status) {
-  constexpr int kKeys = 2 * 257;  // tile count, plus 257 for the chunks of split slots
+  constexpr int kKeys = 3 * 257;  // tile count; + 257: chunks of slots cut in three or more; + 514: in two, paired
   __shared__ int s_len[kMaxPlanBatch];
   __shared__ int s_first[kMaxPlanBatch];
   __shared__ long long s_total;
-  __shared__ int s_chunk, s_entries, s_merges;
+  __shared__ int s_chunk, s_entries, s_merges, s_pairs, s_positions;
   __shared__ int s_hist[kKeys];
   __shared__ int s_base[kKeys];
   const int tid = threadIdx.x;
   if (tid == 0) {
     s_total = 0;
     s_merges = 0;
+    s_positions = 0;
   }
   for (int i = tid; i < kKeys; i += blockDim.x) s_hist[i] = 0;
   for (int i = tid; i < batch * kv_heads; i += blockDim.x) arrivals[i] = 0;
+  for (int i = tid; i < max_entries; i += blockDim.x) entries[i] = PlanEntry{-1, 0, 0, 0, 0, 0, {0, 0}};
   __syncthreads();
   long long mine = 0;
   bool full = false;  // a slot with no room left for the step's token
@@ -156,6 +164,15 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     const int nc = chunks_of(b);
     return nc == 1 ? s_len[b] : ((s_len[b] + nc - 1) / nc + kTile - 1) / kTile * kTile;
   };
+  // Entries of one round of the streaming kernel's walk (see item_index there):
+  // entry e of a round goes, head by head, to workers that differ by the
+  // workgroups' count between e and e + per_round / 2 - the two groups of one
+  // workgroup.  Where that holds, the two chunks of a slot cut in two are put
+  // on such a pair of places: the groups then fold the slot through LDS and it
+  // needs neither partials nor a merge entry.
+  const int per_round = workers / kv_heads;
+  const bool pairing = kv_heads * 16 <= workers && (workers / 16) % kv_heads == 0;
+  auto paired = [&](int b) { return pairing && chunks_of(b) == 2; };
   // a slot's first partial record: running sum of the chunk counts, 256 slots a pass
   {
     int base = 0;
@@ -169,13 +186,19 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     if (tid == 0) s_entries = base;
   }
   __syncthreads();
-  auto key_of = [&](int count, bool split) {
+  // sort keys: paired slots (one key a slot, by its chunk's tiles), then the
+  // chunks of the other cut slots, then whole slots, each longest first
+  auto key_of = [&](int count, int kind) {
     const int tiles = (count + kTile - 1) / kTile;
-    return (tiles > 256 ? 256 : tiles) + (split ? 257 : 0);
+    return (tiles > 256 ? 256 : tiles) + 257 * kind;
   };
   for (int b = tid; b < batch; b += blockDim.x) {
     const int nc = chunks_of(b), cl = chunk_len(b);
-    for (int c = 0; c < nc; ++c) atomicAdd(&s_hist[key_of(min(cl, s_len[b] - c * cl), nc > 1)], 1);
+    if (paired(b)) {
+      atomicAdd(&s_hist[key_of(cl, 2)], 1);
+    } else {
+      for (int c = 0; c < nc; ++c) atomicAdd(&s_hist[key_of(min(cl, s_len[b] - c * cl), nc > 1 ? 1 : 0)], 1);
+    }
   }
   __syncthreads();
   {
@@ -190,25 +213,61 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     }
   }
   __syncthreads();
+  // ranks [0, n_pairs) are the paired slots (keys 514..770 come first)
+  if (tid == 0) {
+    int n = 0;
+    for (int k = 2 * 257; k < kKeys; ++k) n += s_hist[k];
+    s_pairs = n;
+  }
+  __syncthreads();
+  const int n_pairs = s_pairs;
+  const int half = per_round / 2;
+  const int full_rounds = pairing ? n_pairs / half : 0, in_last = pairing ? n_pairs % half : 0;
+  const int holes = in_last > 0 ? half - in_last : 0;  // free places in each half of the pairs' last round
+  // place of the rank-th entry that is not a pair's
+  auto place_of = [&](int rank) {
+    const int base = full_rounds * per_round;
+    if (rank < holes) return base + in_last + rank;
+    if (rank < 2 * holes) return base + half + in_last + (rank - holes);
+    return base + (in_last > 0 ? per_round : 0) + (rank - 2 * holes);
+  };
   for (int b = tid; b < batch; b += blockDim.x) {
     const int nc = chunks_of(b), cl = chunk_len(b), first = s_first[b];
+    if (paired(b)) {
+      const int q = atomicAdd(&s_base[key_of(cl, 2)], 1);
+      const int at = (q / half) * per_round + q % half;
+      // part = -1: folded with its partner through LDS, no partial record
+      if (at + half < max_entries) {
+        entries[at] = PlanEntry{b, 0, cl, -1, 2, s_len[b], {0, 0}};
+        entries[at + half] = PlanEntry{b, cl, s_len[b] - cl, -1, 2, s_len[b], {0, 0}};
+        atomicMax(&s_positions, at + half + 1);
+      }
+      continue;
+    }
     for (int c = 0; c < nc; ++c) {
       const int count = min(cl, s_len[b] - c * cl);
-      const int at = atomicAdd(&s_base[key_of(count, nc > 1)], 1);
-      if (at < max_entries) entries[at] = PlanEntry{b, c * cl, count, first + c, nc, s_len[b], {0, 0}};
-    }
-    if (nc > 1) {  // the slot's merge entry, after every chunk and whole slot
-      const int at = s_entries + atomicAdd(&s_merges, 1);
-      if (at < max_entries) entries[at] = PlanEntry{b, -1, 0, first, nc, s_len[b], {0, 0}};
+      const int at = place_of(atomicAdd(&s_base[key_of(count, nc > 1 ? 1 : 0)], 1) - n_pairs);
+      if (at < max_entries) {
+        entries[at] = PlanEntry{b, c * cl, count, first + c, nc, s_len[b], {0, 0}};
+        atomicMax(&s_positions, at + 1);
+      }
     }
   }
   __syncthreads();
-  for (int i = s_entries + s_merges + tid; i < max_entries; i += blockDim.x)
-    entries[i] = PlanEntry{-1, 0, 0, 0, 0, 0, {0, 0}};
+  // merge entries, one for every slot cut in three or more (or in two where there is no pairing), after the last place
+  const int n_places = min(s_positions, max_entries);
+  for (int b = tid; b < batch; b += blockDim.x) {
+    const int nc = chunks_of(b);
+    if (nc > 1 && !paired(b)) {
+      const int at = n_places + atomicAdd(&s_merges, 1);
+      if (at < max_entries) entries[at] = PlanEntry{b, -1, 0, s_first[b], nc, s_len[b], {0, 0}};
+    }
+  }
+  __syncthreads();
   if (tid < kHandOutCounters) status[kStateHandOut + tid * kStateHandOutStride] = 0;
   if (tid == 0) {
-    status[kStateEntries] = min(s_entries, max_entries);
-    status[kStateMerges] = max(min(s_entries + s_merges, max_entries) - s_entries, 0);
+    status[kStateEntries] = n_places;
+    status[kStateMerges] = max(min(n_places + s_merges, max_entries) - n_places, 0);
   }
 }
 
@@ -254,7 +313,7 @@ int32_t attn_plan_launch(const jpt_attn_args& a, bool paged, hipStream_t stream)
   const int cap = paged ? a.max_pages * a.page_size : a.seq;
   JPT_REQUIRE(cap > 0, "sequence capacity must be positive");
   hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(256), 0, stream, a.lengths, a.batch, cap,
-                     a.kv_heads, target_items(), reinterpret_cast<PlanEntry*>(ws + l.entries),
+                     a.kv_heads, target_items(), persistent_blocks(), reinterpret_cast<PlanEntry*>(ws + l.entries),
                      reinterpret_cast<int32_t*>(ws + l.arrivals), l.max_entries,
                      reinterpret_cast<int32_t*>(ws));
   return launch_status("plan_kernel");

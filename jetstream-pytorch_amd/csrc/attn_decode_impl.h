@@ -383,6 +383,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
   __shared__ int sm_qtaken_all[kGroups][C::kQBufs];   // consumers that took this query buffer
   __shared__ int sm_arrived_all[kGroups][C::kFoldBufs];
   __shared__ int sm_folded_all[kGroups][C::kFoldBufs];
+  __shared__ int sm_pair_ready[C::kFoldBufs];  // items whose parts group 1 has left for group 0 to fold (paired chunks)
   __shared__ int sm_abort;
   __shared__ __attribute__((aligned(16))) int sm_items_all[kGroups][kListedItems][8];
   // page ids of the item being issued and of the next one (paged caches)
@@ -407,6 +408,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
   if (tid < kGroups * C::kFoldBufs) {
     (&sm_arrived_all[0][0])[tid] = 0;
     (&sm_folded_all[0][0])[tid] = 0;
+    if (tid < C::kFoldBufs) sm_pair_ready[tid] = 0;
   }
   if (tid < kGroups * C::kQBufs) (&sm_qtaken_all[0][0])[tid] = 0;
 
@@ -534,11 +536,46 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
     return true;
   };
 
-  // One float written through to memory / read from memory past every cache
-  // level: what workgroups on different XCDs, each behind an L2 of its own,
-  // exchange without a device-wide fence.
-  auto put = [](float* at, float x) { __hip_atomic_store(at, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM); };
-  auto get = [](const float* at) { return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM); };
+  // Partials travel between workgroups on different XCDs, each behind an L2 of
+  // its own, without a device-wide fence: they are written through to memory and
+  // read from memory past every cache level (system scope).  A row of a partial
+  // is written and read 16 bytes a lane with the 16 lanes of a row side by side -
+  // float4 number q of lane l at float 64 q + 4 l, so lane l's outputs
+  // [8 l, 8 l + 8) are its two float4 - because a wave's store of 256 contiguous
+  // bytes is whole memory lines, where one float a lane 32 bytes apart costs a
+  // 32-byte memory write each (measured: 7 MB of writes a launch for 0.7 MB of
+  // partials).  The row's statistics (max, sum) follow at float 128.
+  auto put_row = [](float* row, int lane_in_row, const float (&o)[8], float M, float l) {
+    const f32x4 q0 = {o[0], o[1], o[2], o[3]}, q1 = {o[4], o[5], o[6], o[7]};
+    float* at = row + 4 * lane_in_row;
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\t"
+                 "global_store_dwordx4 %0, %2, off offset:256 sc0 sc1" : : "v"(at), "v"(q0), "v"(q1) : "memory");
+    if (lane_in_row == 0) {
+      typedef __attribute__((ext_vector_type(2))) float f32x2;
+      const f32x2 st = {M, l};
+      asm volatile("global_store_dwordx2 %0, %1, off offset:512 sc0 sc1" : : "v"(row), "v"(st) : "memory");
+    }
+  };
+  // Rows of two partials at once (one memory latency for both); the caller's
+  // wave has no other loads in flight.
+  struct PartRow {
+    f32x4 q0, q1;
+    __attribute__((ext_vector_type(2))) float st;
+  };
+  auto get_rows = [](const float* row_a, const float* row_b, int lane_in_row, PartRow& ra, PartRow& rb) {
+    const float* at_a = row_a + 4 * lane_in_row;
+    const float* at_b = row_b + 4 * lane_in_row;
+    asm volatile("global_load_dwordx4 %0, %6, off sc0 sc1\n\t"
+                 "global_load_dwordx4 %1, %6, off offset:256 sc0 sc1\n\t"
+                 "global_load_dwordx2 %2, %7, off offset:512 sc0 sc1\n\t"
+                 "global_load_dwordx4 %3, %8, off sc0 sc1\n\t"
+                 "global_load_dwordx4 %4, %8, off offset:256 sc0 sc1\n\t"
+                 "global_load_dwordx2 %5, %9, off offset:512 sc0 sc1\n\t"
+                 "s_waitcnt vmcnt(0)"
+                 : "=&v"(ra.q0), "=&v"(ra.q1), "=&v"(ra.st), "=&v"(rb.q0), "=&v"(rb.q1), "=&v"(rb.st)
+                 : "v"(at_a), "v"(row_a), "v"(at_b), "v"(row_b)
+                 : "memory");
+  };
   // writes rows of outputs: 16 lanes a row, eight outputs a lane, the statistics by the row's first lane
   auto write_row = [&](int64_t q_row, int d0, const float (&o)[8], float M, float l) {
     const float inv = l > 0.f ? 1.f / l : 0.f;
@@ -570,41 +607,30 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
     const int64_t step = static_cast<int64_t>(a.kv_heads) * rec;
     const int64_t q_row0 = (static_cast<int64_t>(it.slot) * a.q_heads + it.h * p.rep) * a.q_rows;
     const int d0 = 8 * (lane & 15);
-    constexpr int kBatch = 4;  // chunks loaded together
     for (int row = lane >> 4; row < R; row += 4) {
       const float* src = p.partials + (static_cast<int64_t>(it.part) * a.kv_heads + it.h) * rec + row * kPartFloats;
       float M = -INFINITY, L = 0.f;
       float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      for (int c0 = 0; c0 < it.n_chunks; c0 += kBatch) {
-        float x[kBatch][8], m[kBatch], l[kBatch];
-#pragma unroll
-        for (int c = 0; c < kBatch; ++c) {
-          m[c] = -INFINITY;
-          l[c] = 0.f;
-          if (c0 + c < it.n_chunks) {
-            const float* s = src + (c0 + c) * step;
-            m[c] = get(s + kD);
-            l[c] = get(s + kD + 1);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) x[c][i] = get(s + d0 + i);
-          } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) x[c][i] = 0.f;
-          }
-        }
-        float Mb = M;
-#pragma unroll
-        for (int c = 0; c < kBatch; ++c) Mb = fmaxf(Mb, m[c]);
+      for (int c0 = 0; c0 < it.n_chunks; c0 += 2) {  // two chunks a trip to memory
+        const bool two = c0 + 1 < it.n_chunks;
+        PartRow x[2];
+        get_rows(src + c0 * step, src + (two ? c0 + 1 : c0) * step, lane & 15, x[0], x[1]);
+        const float m0 = x[0].st[0], m1 = two ? x[1].st[0] : -INFINITY;
+        const float Mb = fmaxf(M, fmaxf(m0, m1));
         const float keep_old = M == -INFINITY ? 0.f : fast_exp2(M - Mb);
         L *= keep_old;
 #pragma unroll
         for (int i = 0; i < 8; ++i) o[i] *= keep_old;
 #pragma unroll
-        for (int c = 0; c < kBatch; ++c) {
-          const float f = m[c] == -INFINITY ? 0.f : fast_exp2(m[c] - Mb);
-          L += l[c] * f;
+        for (int c = 0; c < 2; ++c) {
+          const float mc = c == 0 ? m0 : m1;
+          const float f = mc == -INFINITY ? 0.f : fast_exp2(mc - Mb);
+          L += x[c].st[1] * f;
 #pragma unroll
-          for (int i = 0; i < 8; ++i) o[i] += x[c][i] * f;
+          for (int i = 0; i < 4; ++i) {
+            o[i] += x[c].q0[i] * f;
+            o[4 + i] += x[c].q1[i] * f;
+          }
         }
         M = Mb;
       }
@@ -1265,42 +1291,60 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
     arrived = __builtin_amdgcn_readfirstlane(arrived);
     if (arrived != kConsumers - 1) return true;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    // Paired chunks (part < 0): the two chunks of a slot cut in two run on the
+    // two groups of this workgroup, as the same item of both (the planner puts
+    // them on the same round, and every round before it is full).  Group 1
+    // leaves its consumers' parts in its fold buffer and says so; group 0 folds
+    // both groups' parts, writes the slot's output and frees both buffers.
+    const bool pair = it.n_chunks > 1 && it.part < 0;
+    if (pair && group == 1) {
+      if (lane == 0) __hip_atomic_store(&sm_pair_ready[buf], seq + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      return true;
+    }
+    if (pair && !wait_for(&sm_pair_ready[buf], seq + 1)) return false;
     const int64_t q_row0 = (static_cast<int64_t>(it.slot) * a.q_heads + it.h * p.rep) * a.q_rows;
-    float* part = p.partials + (static_cast<int64_t>(it.part) * a.kv_heads + it.h) * R * kPartFloats;
+    float* part = p.partials + (static_cast<int64_t>(pair ? 0 : it.part) * a.kv_heads + it.h) * R * kPartFloats;
     // four rows a pass: 16 lanes a row, eight consecutive outputs a lane
     const int d0 = 8 * (lane & 15);
+    const int n_groups = pair ? 2 : 1;  // whose parts are folded: this group's, then (paired) group 1's
     for (int row = lane >> 4; row < R; row += 4) {
       float M = -INFINITY;
+      for (int gi = 0; gi < n_groups; ++gi) {
+        const auto& mm = sm_m_all[gi == 0 ? group : 1];
 #pragma unroll
-      for (int w2 = 0; w2 < kConsumers; ++w2) M = fmaxf(M, sm_m[buf][w2][row]);
+        for (int w2 = 0; w2 < kConsumers; ++w2) M = fmaxf(M, mm[buf][w2][row]);
+      }
       float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       float l = 0.f;
+      for (int gi = 0; gi < n_groups; ++gi) {
+        const auto& mm = sm_m_all[gi == 0 ? group : 1];
+        const auto& ll = sm_l_all[gi == 0 ? group : 1];
+        const auto& oo = sm_o_all[gi == 0 ? group : 1];
 #pragma unroll
-      for (int w2 = 0; w2 < kConsumers; ++w2) {
-        const float mw = sm_m[buf][w2][row];
-        const float f = mw == -INFINITY ? 0.f : fast_exp2(mw - M);
-        l += sm_l[buf][w2][row] * f;
-        const float4* src = reinterpret_cast<const float4*>(&sm_o[buf][w2][row][o_col(d0)]);
-        const float4 x = src[0], y = src[1];
-        o[0] += x.x * f; o[1] += x.y * f; o[2] += x.z * f; o[3] += x.w * f;
-        o[4] += y.x * f; o[5] += y.y * f; o[6] += y.z * f; o[7] += y.w * f;
-      }
-      if (it.n_chunks == 1) {
-        write_row(q_row0 + row, d0, o, M, l);
-      } else {  // park the chunk's partial where the workgroups of every XCD see it
-        float* dst = part + row * kPartFloats;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) put(dst + d0 + i, o[i]);
-        if (d0 == 0) {
-          put(dst + kD, M);
-          put(dst + kD + 1, l);
+        for (int w2 = 0; w2 < kConsumers; ++w2) {
+          const float mw = mm[buf][w2][row];
+          const float f = mw == -INFINITY ? 0.f : fast_exp2(mw - M);
+          l += ll[buf][w2][row] * f;
+          const float4* src = reinterpret_cast<const float4*>(&oo[buf][w2][row][o_col(d0)]);
+          const float4 x = src[0], y = src[1];
+          o[0] += x.x * f; o[1] += x.y * f; o[2] += x.z * f; o[3] += x.w * f;
+          o[4] += y.x * f; o[5] += y.y * f; o[6] += y.z * f; o[7] += y.w * f;
         }
       }
+      if (it.n_chunks == 1 || pair) {
+        write_row(q_row0 + row, d0, o, M, l);
+      } else {  // park the chunk's partial where the workgroups of every XCD see it
+        put_row(part + row * kPartFloats, lane & 15, o, M, l);
+      }
     }
-    if (it.n_chunks > 1) owed_arrival = p.arrivals + static_cast<int64_t>(it.slot) * a.kv_heads + it.h;
+    if (it.n_chunks > 1 && !pair) owed_arrival = p.arrivals + static_cast<int64_t>(it.slot) * a.kv_heads + it.h;
     if (lane == 0) {
       __hip_atomic_store(&sm_arrived[buf], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       __hip_atomic_fetch_add(&sm_folded[buf], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (pair) {
+        __hip_atomic_store(&sm_arrived_all[1][buf], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        __hip_atomic_fetch_add(&sm_folded_all[1][buf], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
     }
     return true;
   };

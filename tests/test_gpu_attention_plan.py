@@ -1,0 +1,112 @@
+"""The decode-attention plan, read back from the workspace.  The streaming
+kernel trusts the planner's records (it never checks one), so the properties
+it relies on are checked here on the planner's own output: whatever the
+lengths, the work entries cover every position of every slot exactly once;
+the two chunks of a slot cut in two sit on places that one workgroup's two
+groups walk in the same round, with every earlier round full; every other cut
+slot has consecutive partial records and one merge entry that names them all.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+TILE = 32
+STATE_BYTES = 64 * 1024
+ENTRY_INTS = 8  # slot, start, count, part, n_chunks, slot_len, unused, unused
+
+
+def workers():
+  cus = torch.cuda.get_device_properties(0).multi_processor_count
+  return (cus * 2 + 7) // 8 * 8
+
+
+def read_plan(plan):
+  """(work places incl. unused ones, merge entries) as numpy int32 [n, 8]."""
+  torch.cuda.synchronize()
+  raw = plan.workspace.buf.cpu().numpy()
+  state = raw[:STATE_BYTES].view(np.int32)
+  n_places, n_merges = int(state[2]), int(state[3])
+  entries = raw[STATE_BYTES:STATE_BYTES + (n_places + n_merges) * ENTRY_INTS * 4].view(np.int32).reshape(-1, ENTRY_INTS)
+  return entries[:n_places], entries[n_places:]
+
+
+def check_plan(lengths, kv_heads, seq):
+  from jetstream_pt_amd import attention_kernel as ak
+  batch = len(lengths)
+  dl = torch.tensor(lengths, dtype=torch.int32, device=DEV)
+  plan = ak.DecodePlan(dl, batch, kv_heads * 4, kv_heads, seq=seq)
+  places, merges = read_plan(plan)
+  clipped = [min(max(n, 0), seq) for n in lengths]
+  per_round = workers() // kv_heads
+  pairing = kv_heads * 16 <= workers() and (workers() // 16) % kv_heads == 0
+  covered = [np.zeros(n, dtype=np.int32) for n in clipped]
+  chunks = [[] for _ in range(batch)]
+  for at, (slot, start, count, part, n_chunks, slot_len, _, _) in enumerate(places):
+    if slot < 0:
+      continue  # a place nobody was put on
+    assert 0 <= slot < batch and slot_len == clipped[slot]
+    assert start >= 0 and start % TILE == 0 and start + count <= slot_len
+    assert count > 0 or slot_len == 0
+    covered[slot][start:start + count] += 1
+    chunks[slot].append((start, count, part, n_chunks, at))
+  merge_of = {}
+  for slot, start, count, part, n_chunks, slot_len, _, _ in merges:
+    assert start == -1 and slot not in merge_of
+    merge_of[slot] = (part, n_chunks)
+  used_parts = set()
+  n_pairs = 0
+  for slot in range(batch):
+    assert np.all(covered[slot] == 1), slot
+    cs = sorted(chunks[slot])
+    assert len(cs) >= 1  # an empty slot still has an item that writes its output
+    assert all(c[3] == len(cs) for c in cs)
+    if len(cs) == 1:
+      assert slot not in merge_of
+      continue
+    assert all(c[1] >= 1 for c in cs)
+    if pairing and len(cs) == 2:
+      # folded through LDS by the two groups of one workgroup: same round, half a round apart, no partials
+      n_pairs += 1
+      (s0, c0, p0, _, at0), (s1, c1, p1, _, at1) = cs
+      assert p0 == -1 and p1 == -1 and slot not in merge_of
+      assert at1 == at0 + per_round // 2 and at0 % per_round < per_round // 2
+      # the item has the same number in both groups' walks: every place of the rounds before is taken
+      assert np.all(places[:at0 // per_round * per_round, 0] >= 0)
+      continue
+    part0, n = merge_of[slot]
+    assert n == len(cs)
+    assert [c[2] for c in cs] == list(range(part0, part0 + n)), "partials numbered along the slot"
+    assert not used_parts & set(range(part0, part0 + n))
+    used_parts |= set(range(part0, part0 + n))
+  assert len(merge_of) == sum(1 for s in range(batch) if len(chunks[s]) > 1) - n_pairs
+  return n_pairs, len(merge_of)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_plan_covers_every_position_once_lognormal(seed):
+  rng = np.random.default_rng(seed)
+  lengths = [int(x) for x in np.clip(np.round(np.exp(np.log(400) + rng.standard_normal(128))), 16, 8192)]
+  n_pairs, n_merges = check_plan(lengths, 8, 8192)
+  assert n_pairs + n_merges > 0  # the distribution's tail is cut
+
+
+@pytest.mark.parametrize("lengths,kv_heads,seq", [
+    ([0], 1, 64),                       # one empty slot
+    ([1], 1, 64),
+    ([64], 8, 64),
+    ([4096], 1, 4096),                  # one slot in many chunks
+    ([4096, 3000, 1, 0, 17, 2049] * 4, 8, 4096),
+    ([0] * 40, 4, 256),                 # nothing but empty slots
+    ([33] * 700, 2, 64),                # many short slots, several rounds
+    ([5000, -3, 70], 2, 2048),          # out-of-range lengths are clipped
+    ([1024] * 8, 32, 1024),             # every slot cut in two: pairs only
+    ([1024] * 8 + [100] * 3, 32, 1024), # pairs, and whole slots in the places they leave
+    ([2048] * 40, 8, 2048),             # more pairs than one round holds
+    ([1024] * 4096, 2, 1024),           # the largest batch the planner takes
+    ([700] * 5, 3, 1024),               # a head count the workers do not divide by: no pairing
+])
+def test_plan_covers_every_position_once_edge_cases(lengths, kv_heads, seq):
+  check_plan(lengths, kv_heads, seq)
