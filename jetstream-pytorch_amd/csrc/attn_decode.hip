@@ -132,6 +132,7 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     s_total = 0;
     s_merges = 0;
     s_positions = 0;
+    s_pairs = 0;
   }
   for (int i = tid; i < kKeys; i += blockDim.x) s_hist[i] = 0;
   for (int i = tid; i < batch * kv_heads; i += blockDim.x) arrivals[i] = 0;
@@ -196,6 +197,7 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     const int nc = chunks_of(b), cl = chunk_len(b);
     if (paired(b)) {
       atomicAdd(&s_hist[key_of(cl, 2)], 1);
+      atomicAdd(&s_pairs, 1);
     } else {
       for (int c = 0; c < nc; ++c) atomicAdd(&s_hist[key_of(min(cl, s_len[b] - c * cl), nc > 1 ? 1 : 0)], 1);
     }
@@ -213,14 +215,7 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     }
   }
   __syncthreads();
-  // ranks [0, n_pairs) are the paired slots (keys 514..770 come first)
-  if (tid == 0) {
-    int n = 0;
-    for (int k = 2 * 257; k < kKeys; ++k) n += s_hist[k];
-    s_pairs = n;
-  }
-  __syncthreads();
-  const int n_pairs = s_pairs;
+  const int n_pairs = s_pairs;  // ranks [0, n_pairs) are the paired slots (their keys come first)
   const int half = per_round / 2;
   const int full_rounds = pairing ? n_pairs / half : 0, in_last = pairing ? n_pairs % half : 0;
   const int holes = in_last > 0 ? half - in_last : 0;  // free places in each half of the pairs' last round
