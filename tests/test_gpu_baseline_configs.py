@@ -40,11 +40,16 @@ def as_np(x):
   return x.cpu().numpy() if isinstance(x, torch.Tensor) else np.asarray(x)
 
 
-def close(got, want, name, extra=None):
-  """|got - want| <= 1e-2 + 2^-8 |want| (+ extra, a tensor broadcastable to them)."""
+def close(got, want, name, extra=None, pure=False):
+  """|got - want| <= 1e-2 + 2^-8 |want| (+ extra, a tensor broadcastable to them).
+  The second term is the half ulp by which a bf16 output differs from the
+  unrounded expectation; `pure`: outputs small enough that max-abs 1e-2 holds
+  without it."""
   got, want = got.double().cpu(), want.double()
   err = record_parity(name, got, want)
   bound = ATOL + RTOL * want.abs()
+  if pure:
+    bound = torch.full_like(want, ATOL)
   if extra is not None:
     bound = bound + extra
   bad = err > bound
@@ -78,7 +83,7 @@ def test_c1_dense_bf16_eager_update_and_attention():
     want[b.to(want.device), :, pos.to(want.device), :] = new[:, :, 0, :]
     assert torch.equal(after, want)
   want, _, _ = oattn.closed_form(w["xq"].cpu(), cache.cache_k.cpu(), cache.cache_v.cpu(), mask=w["mask"].cpu())
-  close(out, want, "c1/closed_form")
+  close(out, want, "c1/closed_form", pure=True)
 
 
 def dense_int8_step_checks(w, batch, hkv, name):
@@ -90,12 +95,12 @@ def dense_int8_step_checks(w, batch, hkv, name):
   torch.cuda.synchronize()
   # the lazy stash of layer 0: codes and scales of the decode quantiser, computed in float32
   stash = {}
-  for name, x, codes, scale in (("k", w["xk"], cache.new_ks[0], cache.new_k_scaler[0]),
-                                ("v", w["xv"], cache.new_vs[0], cache.new_v_scaler[0])):
+  for which, x, codes, scale in (("k", w["xk"], cache.new_ks[0], cache.new_k_scaler[0]),
+                                 ("v", w["xv"], cache.new_vs[0], cache.new_v_scaler[0])):
     want_c, want_s = oquant.quantize_decode(x.cpu(), compute_dtype=torch.float32)
-    assert torch.equal(codes.cpu().reshape(want_c.shape), want_c), name
-    assert torch.equal(scale.cpu().reshape(-1), want_s.reshape(-1)), name
-    stash[name] = (codes.clone(), scale.clone())
+    assert torch.equal(codes.cpu().reshape(want_c.shape), want_c), which
+    assert torch.equal(scale.cpu().reshape(-1), want_s.reshape(-1)), which
+    stash[which] = (codes.clone(), scale.clone())
   # attention over cache + merged new token against the oracle's layer kernel
   oenv = OEnv(batch_size=batch, num_layers=1, ring_buffer=False)
   ocache = okv.Int8KVCacheGenerate.empty((1, batch, hkv, cache.cache_k.shape[3], bench.D), None, oenv,
