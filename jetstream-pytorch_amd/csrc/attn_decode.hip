@@ -50,6 +50,8 @@ struct Layout {
 
 constexpr int kMaxPlanBatch = 4096;
 constexpr int kMaxChunksPerSlot = 256;
+constexpr int kMaxBins = 1024;         // entries of one round of the workers' walk: workers / kv_heads
+constexpr int kDealtOneByOne = 512;  // entries dealt to the lightest bin one by one (about 0.12 us each)
 
 // Workers of the streaming kernel: two groups of waves on every compute unit.
 int32_t persistent_blocks() {
@@ -74,7 +76,9 @@ Layout make_layout(int batch, int kv_heads, int rows) {
   // and every split slot has at least one), and a merge entry for each split slot
   const int extra = (target_items() + kv_heads - 1) / kv_heads + 1;
   // ... and the places a half-filled round of paired chunks leaves empty
-  l.max_entries = (batch + 2 * extra + persistent_blocks() / kv_heads + 8 + 7) / 8 * 8;
+  // Every bin (workers / kv_heads of them) may end one round short of the fullest: two rounds of
+  // slack, and up to `batch` merge entries behind the places.
+  l.max_entries = (2 * batch + 2 * extra + 3 * (persistent_blocks() / kv_heads + 8) + 7) / 8 * 8;
   auto up = [](int64_t x) { return (x + 255) / 256 * 256; };
   l.entries = JPT_ATTN_WS_STATE_BYTES;
   l.arrivals = up(l.entries + static_cast<int64_t>(l.max_entries) * sizeof(PlanEntry));
@@ -117,6 +121,83 @@ __device__ __forceinline__ int plan_exclusive_scan(int x, int* total) {
   return before + incl - x;
 }
 
+// Minimum of `x` over the wave, the same (scalar) value for every lane: within the
+// 16-lane rows by data-parallel primitives, across the four rows by lane reads.
+template <int CTRL>
+__device__ __forceinline__ unsigned plan_dpp(unsigned v) {
+  return static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ unsigned wave_min_u32(unsigned x) {
+  x = min(x, plan_dpp<0xB1>(x));   // quad_perm [1, 0, 3, 2]
+  x = min(x, plan_dpp<0x4E>(x));   // quad_perm [2, 3, 0, 1]
+  x = min(x, plan_dpp<0x141>(x));  // row_half_mirror
+  x = min(x, plan_dpp<0x140>(x));  // row_mirror
+  const int v = static_cast<int>(x);
+  const unsigned a = static_cast<unsigned>(__builtin_amdgcn_readlane(v, 0)), b = static_cast<unsigned>(__builtin_amdgcn_readlane(v, 16));
+  const unsigned c = static_cast<unsigned>(__builtin_amdgcn_readlane(v, 32)), d = static_cast<unsigned>(__builtin_amdgcn_readlane(v, 48));
+  return min(min(a, b), min(c, d));
+}
+
+// Longest-processing-time deal by one wave.  Entry `rank` (longest first, its
+// tiles in rank_tiles) goes to the bin with the fewest tiles so far, into the
+// bin's first free round; rank_place gets its place.  Everything lives in
+// registers: lane l keeps bins l, l + 64, ... as (tiles << 10 | bin), and the
+// tiles and places of the 64 ranks of the current block, one a lane; the loop
+// body is a wave-wide minimum, two lane reads and a few selects, with no memory
+// access and no branch (an entry costs about a quarter of a microsecond less
+// than with LDS in the loop, and there are hundreds).
+template <int PER_LANE>
+__device__ __forceinline__ void deal_longest_first(int n, int per_round, int max_rounds, int* bin_load,
+                                                   int* bin_rounds, const int* rank_tiles, int* rank_place) {
+  const int lane = threadIdx.x;
+  unsigned mine[PER_LANE];
+  int rounds[PER_LANE];
+#pragma unroll
+  for (int i = 0; i < PER_LANE; ++i) {
+    const int x = lane + 64 * i;
+    rounds[i] = x < per_round ? bin_rounds[x] : max_rounds;
+    // a bin with no free round is out of the running (there is room for all: max_rounds * per_round)
+    mine[i] = rounds[i] < max_rounds ? (static_cast<unsigned>(bin_load[x]) << 10) | static_cast<unsigned>(x) : ~0u;
+  }
+  for (int block = 0; block < n; block += 64) {
+    const int my_tiles = block + lane < n ? rank_tiles[block + lane] : 0;
+    int my_place = 0;
+    const int in_block = min(64, n - block);
+    for (int j = 0; j < in_block; ++j) {
+      const unsigned tiles = static_cast<unsigned>(__builtin_amdgcn_readlane(my_tiles, j));
+      unsigned best = mine[0];
+#pragma unroll
+      for (int i = 1; i < PER_LANE; ++i) best = min(best, mine[i]);
+      best = wave_min_u32(best);
+      const int x = static_cast<int>(best & 1023u);
+      int round = 0;
+#pragma unroll
+      for (int i = 0; i < PER_LANE; ++i) {
+        const bool here = PER_LANE == 1 || (x >> 6) == i;  // wave-uniform
+        if (here) round = __builtin_amdgcn_readlane(rounds[i], x & 63);
+      }
+      const int place = round * per_round + ((round & 1) ? per_round - 1 - x : x);
+      const bool winner = (x & 63) == lane;
+#pragma unroll
+      for (int i = 0; i < PER_LANE; ++i) {
+        const bool here = winner && (PER_LANE == 1 || (x >> 6) == i);
+        rounds[i] += here ? 1 : 0;
+        mine[i] = !here ? mine[i] : rounds[i] < max_rounds ? mine[i] + (tiles << 10) : ~0u;
+      }
+      my_place = lane == j ? place : my_place;
+    }
+    if (block + lane < n) rank_place[block + lane] = my_place;
+  }
+#pragma unroll
+  for (int i = 0; i < PER_LANE; ++i) {
+    const int x = lane + 64 * i;
+    if (x < per_round) {
+      bin_rounds[x] = rounds[i];
+      bin_load[x] = static_cast<int>(mine[i] >> 10);  // a full bin reads as the heaviest, which suits what follows
+    }
+  }
+}
+
 __global__ void __launch_bounds__(256)
 plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int target, int workers,
             PlanEntry* entries, int32_t* arrivals, int max_entries, int32_t* status) {
@@ -124,15 +205,20 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
   __shared__ int s_len[kMaxPlanBatch];
   __shared__ int s_first[kMaxPlanBatch];
   __shared__ long long s_total;
-  __shared__ int s_chunk, s_entries, s_merges, s_pairs, s_positions;
+  __shared__ int s_chunk, s_entries, s_merges, s_pairs, s_positions, s_sizes;
   __shared__ int s_hist[kKeys];
   __shared__ int s_base[kKeys];
+  __shared__ int s_bin_load[kMaxBins];       // tiles dealt to a bin (the workers that take one entry's heads)
+  __shared__ int s_bin_rounds[kMaxBins];     // rounds of the bin that are taken
+  __shared__ int s_rank_tiles[kDealtOneByOne];
+  __shared__ int s_rank_place[kDealtOneByOne];
   const int tid = threadIdx.x;
   if (tid == 0) {
     s_total = 0;
     s_merges = 0;
     s_positions = 0;
     s_pairs = 0;
+    s_sizes = 0;
   }
   for (int i = tid; i < kKeys; i += blockDim.x) s_hist[i] = 0;
   for (int i = tid; i < batch * kv_heads; i += blockDim.x) arrivals[i] = 0;
@@ -172,7 +258,7 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
   // on such a pair of places: the groups then fold the slot through LDS and it
   // needs neither partials nor a merge entry.
   const int per_round = workers / kv_heads;
-  const bool pairing = kv_heads * 16 <= workers && (workers / 16) % kv_heads == 0;
+  const bool pairing = per_round <= kMaxBins && kv_heads * 16 <= workers && (workers / 16) % kv_heads == 0;
   auto paired = [&](int b) { return pairing && chunks_of(b) == 2; };
   // a slot's first partial record: running sum of the chunk counts, 256 slots a pass
   {
@@ -203,6 +289,9 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     }
   }
   __syncthreads();
+  // how many different sizes the entries that are not a pair's have
+  for (int key = tid; key < 2 * 257; key += blockDim.x)
+    if (s_hist[key] > 0) atomicAdd(&s_sizes, 1);
   {
     // where each key's entries start, largest key first: thread t of pass i has key kKeys - 1 - (256 i + t)
     int base = 0;
@@ -217,14 +306,68 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
   __syncthreads();
   const int n_pairs = s_pairs;  // ranks [0, n_pairs) are the paired slots (their keys come first)
   const int half = per_round / 2;
-  const int full_rounds = pairing ? n_pairs / half : 0, in_last = pairing ? n_pairs % half : 0;
-  const int holes = in_last > 0 ? half - in_last : 0;  // free places in each half of the pairs' last round
+  // The deal.  A bin is the set of workers that take the heads of one entry of a
+  // round; bin x has place x of even rounds and place per_round - 1 - x of odd
+  // ones (the streaming kernel walks odd rounds backwards).  Pairs fill rounds
+  // from the first, places x and x + half.  The other entries are dealt longest
+  // first, each to the bin that holds the fewest tiles so far, into that bin's
+  // first free round (longest-processing-time dealing, by one wave: see
+  // deal_longest_first).  `regular`: the walk has whole entries per round, i.e.
+  // bins exist; otherwise entries lie in sorted order.
+  const bool regular = per_round >= 1 && per_round <= kMaxBins && workers % 8 == 0 && (workers / 8) % kv_heads == 0;
+  const int n_others = s_entries - 2 * n_pairs;
+  // (when all of them are equally long there is nothing to even out: they go round the bins)
+  const int one_by_one = regular && s_sizes > 1 ? min(n_others, kDealtOneByOne) : 0;
+  auto bin_of_place = [&](int round, int x) { return (round & 1) ? per_round - 1 - x : x; };
+  const int max_rounds = regular ? max((max_entries - batch) / per_round, 1) : 0;  // up to `batch` merge entries follow the places
+  if (regular) {
+    for (int x = tid; x < per_round; x += blockDim.x) {
+      s_bin_load[x] = 0;
+      s_bin_rounds[x] = 0;
+    }
+    __syncthreads();
+    // tiles of the entries by rank (a key is a tile count; ranks go down the keys), pairs' loads and rounds
+    for (int rank = tid; rank < n_pairs + one_by_one; rank += blockDim.x) {
+      int lo = 0, hi = kKeys - 1;  // the smallest key whose entries start at or before this rank
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (s_base[mid] <= rank) hi = mid; else lo = mid + 1;
+      }
+      const int tiles = lo % 257;
+      if (rank < n_pairs) {  // a pair: both its bins get the chunk's tiles
+        const int round = rank / half, x = rank % half;
+        atomicAdd(&s_bin_load[bin_of_place(round, x)], tiles);
+        atomicAdd(&s_bin_load[bin_of_place(round, x + half)], tiles);
+        atomicMax(&s_bin_rounds[bin_of_place(round, x)], round + 1);
+        atomicMax(&s_bin_rounds[bin_of_place(round, x + half)], round + 1);
+      } else if (rank - n_pairs < one_by_one) {
+        s_rank_tiles[rank - n_pairs] = tiles;
+      }
+    }
+    __syncthreads();
+    // bins the pairs left behind start at the pairs' last full round, so that every round before a pair's is full
+    if (pairing && n_pairs > 0)
+      for (int x = tid; x < per_round; x += blockDim.x) s_bin_rounds[x] = max(s_bin_rounds[x], n_pairs / half);
+    __syncthreads();
+    // Entries beyond the first kDealtOneByOne (only large batches have them, and
+    // they are the short ones) go round the bins in snake order, each into its
+    // bin's next free round.
+    const int laps_after = (n_others - one_by_one + per_round - 1) / per_round;
+    if (tid < 64 && one_by_one > 0) {
+      const int cap = max(max_rounds - laps_after, 1);
+      if (per_round <= 64) deal_longest_first<1>(one_by_one, per_round, cap, s_bin_load, s_bin_rounds, s_rank_tiles, s_rank_place);
+      else if (per_round <= 256) deal_longest_first<4>(one_by_one, per_round, cap, s_bin_load, s_bin_rounds, s_rank_tiles, s_rank_place);
+      else deal_longest_first<16>(one_by_one, per_round, cap, s_bin_load, s_bin_rounds, s_rank_tiles, s_rank_place);
+    }
+    __syncthreads();
+  }
   // place of the rank-th entry that is not a pair's
   auto place_of = [&](int rank) {
-    const int base = full_rounds * per_round;
-    if (rank < holes) return base + in_last + rank;
-    if (rank < 2 * holes) return base + half + in_last + (rank - holes);
-    return base + (in_last > 0 ? per_round : 0) + (rank - 2 * holes);
+    if (!regular) return rank;  // no pairs either
+    if (rank < one_by_one) return s_rank_place[rank];
+    const int i = rank - one_by_one, lap = i / per_round, x = (lap & 1) ? per_round - 1 - i % per_round : i % per_round;
+    const int round = s_bin_rounds[x] + lap;  // one entry a bin and lap
+    return round * per_round + bin_of_place(round, x);
   };
   for (int b = tid; b < batch; b += blockDim.x) {
     const int nc = chunks_of(b), cl = chunk_len(b), first = s_first[b];
