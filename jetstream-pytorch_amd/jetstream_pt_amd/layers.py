@@ -20,6 +20,7 @@ import torch
 
 from . import _ffi
 from . import attention_kernel as ak
+from .scopes import scoped
 from .cache_manager import Int8KVCacheGenerate
 
 
@@ -113,21 +114,21 @@ class AttentionKernel:
     seqlen = xq.shape[2]
     args = (cache, start, end, ragged_batch_index, ragged_block_index)
     if hasattr(cache, "page_attention_manager") and self._will_append_in_launch(xq, cache, cache.cache_k):
-      keys, values = cache.update(xk, xv, self.layer_id, defer_append=True)
+      keys, values = scoped("attn_insert_cache", cache.update, xk, xv, self.layer_id, defer_append=True)
       new = dict(new_key=xk.to(keys.dtype).contiguous(), new_value=xv.to(keys.dtype).contiguous())
-      return self._attend(xq, keys, values, None, None, mask, *args, new_token=new)[0]
-    orig_keys, orig_values = cache.update(xk, xv, self.layer_id)
+      return scoped("attn_qkv+attn_new_qkv+attn_global", self._attend, xq, keys, values, None, None, mask, *args, new_token=new)[0]
+    orig_keys, orig_values = scoped("attn_insert_cache", cache.update, xk, xv, self.layer_id)
     if self._will_fuse(seqlen, orig_keys):
       dt = orig_keys.dtype
       new = dict(new_key=xk.to(dt).contiguous(), new_value=xv.to(dt).contiguous())
-      return self._attend(xq, orig_keys, orig_values, None, None, mask, *args, new_token=new)[0]
-    existing_output, (existing_max, existing_denom) = self._attend(
-        xq, orig_keys, orig_values, None, None, mask, *args)
+      return scoped("attn_qkv+attn_new_qkv+attn_global", self._attend, xq, orig_keys, orig_values, None, None, mask, *args, new_token=new)[0]
+    existing_output, (existing_max, existing_denom) = scoped(
+        "attn_qkv", self._attend, xq, orig_keys, orig_values, None, None, mask, *args)
     if not self.env.lazy_cache_update or seqlen > 1:
       return existing_output
-    new_output, (new_max, new_denom) = self._attend(xq, xk, xv, None, None, None, *args)
-    return ak.lse_merge(existing_output, existing_max, existing_denom, new_output, new_max,
-                        new_denom)
+    new_output, (new_max, new_denom) = scoped("attn_new_qkv", self._attend, xq, xk, xv, None, None, None, *args)
+    return scoped("attn_global", ak.lse_merge, existing_output, existing_max, existing_denom, new_output,
+                  new_max, new_denom)
 
 
 class Int8KVAttentionKernel(AttentionKernel):
@@ -152,7 +153,7 @@ class Int8KVAttentionKernel(AttentionKernel):
         and self._will_append_in_launch(xq, cache, cache.cache_k) and xk.dtype == torch.bfloat16):
       # int8 pages: the attention launch quantises the token, writes codes and
       # scales into its page and attends it
-      keys, values, k_scaler, v_scaler = cache.update(xk, xv, self.layer_id, defer_append=True)
+      keys, values, k_scaler, v_scaler = scoped("attn_insert_cache", cache.update, xk, xv, self.layer_id, defer_append=True)
       bsz, hkv, _, dim = xk.shape
       hs = k_scaler.shape[0]
       new = dict(new_key=torch.empty((bsz, hkv, 1, dim), dtype=torch.int8, device=xk.device),
@@ -161,13 +162,13 @@ class Int8KVAttentionKernel(AttentionKernel):
                  new_v_scaler=torch.empty((bsz, hs), dtype=k_scaler.dtype, device=xk.device),
                  new_key_raw=xk.contiguous(), new_value_raw=xv.contiguous(), new_rounding=cache.rounding,
                  new_key_rope=freqs_cis)
-      return self._attend(xq, keys, values, k_scaler, v_scaler, mask, *args, new_token=new)[0]
+      return scoped("attn_qkv+attn_new_qkv+attn_global", self._attend, xq, keys, values, k_scaler, v_scaler, mask, *args, new_token=new)[0]
     # the ragged launch can quantise the token itself (one launch less)
     fuse_quant = (self.fuse_quantize and isinstance(cache, Int8KVCacheGenerate)
                   and self._will_fuse(seqlen, cache.cache_k) and xk.dtype == torch.bfloat16
                   and xk.is_contiguous() and xv.is_contiguous())
-    ret = cache.update(xk, xv, self.layer_id, defer_quantize=True) if fuse_quant \
-        else cache.update(xk, xv, self.layer_id, **rope_kw)
+    ret = scoped("attn_insert_cache", cache.update, xk, xv, self.layer_id, defer_quantize=True) if fuse_quant \
+        else scoped("attn_insert_cache", cache.update, xk, xv, self.layer_id, **rope_kw)
     if len(ret) == 4:  # int8 pages: (codes k, codes v, scale pages k, scale pages v)
       orig_keys, orig_values, k_scaler, v_scaler = ret
       new_key = new_value = new_k_scaler = new_v_scaler = None
@@ -179,14 +180,14 @@ class Int8KVAttentionKernel(AttentionKernel):
                  new_v_scaler=new_v_scaler)
       if fuse_quant:
         new.update(new_key_raw=xk, new_value_raw=xv, new_rounding=cache.rounding, new_key_rope=freqs_cis)
-      return self._attend(xq, orig_keys, orig_values, k_scaler, v_scaler, mask, *args,
-                          new_token=new)[0]
-    existing_output, (existing_max, existing_denom) = self._attend(
-        xq, orig_keys, orig_values, k_scaler, v_scaler, mask, *args)
+      return scoped("attn_qkv+attn_new_qkv+attn_global", self._attend, xq, orig_keys, orig_values, k_scaler,
+                    v_scaler, mask, *args, new_token=new)[0]
+    existing_output, (existing_max, existing_denom) = scoped(
+        "attn_qkv", self._attend, xq, orig_keys, orig_values, k_scaler, v_scaler, mask, *args)
     if not self.env.lazy_cache_update or seqlen > 1:
       return existing_output
     # over the QUANTISED new token, as the reference does (layers.py:704-706)
-    new_output, (new_max, new_denom) = self._attend(
-        xq, new_key, new_value, new_k_scaler, new_v_scaler, None, *args)
-    return ak.lse_merge(existing_output, existing_max, existing_denom, new_output, new_max,
-                        new_denom)
+    new_output, (new_max, new_denom) = scoped(
+        "attn_new_qkv", self._attend, xq, new_key, new_value, new_k_scaler, new_v_scaler, None, *args)
+    return scoped("attn_global", ak.lse_merge, existing_output, existing_max, existing_denom, new_output,
+                  new_max, new_denom)
