@@ -210,6 +210,8 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
   __shared__ int s_base[kKeys];
   __shared__ int s_bin_load[kMaxBins];       // tiles dealt to a bin (the workers that take one entry's heads)
   __shared__ int s_bin_rounds[kMaxBins];     // rounds of the bin that are taken
+  __shared__ int s_snake_load[kMaxBins];     // the entries a plain snake deal would add to a bin (pairs aside)
+  __shared__ int s_snake_max, s_snake_sum;
   __shared__ int s_rank_tiles[kDealtOneByOne];
   __shared__ int s_rank_place[kDealtOneByOne];
   const int tid = threadIdx.x;
@@ -317,17 +319,20 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
   const bool regular = per_round >= 1 && per_round <= kMaxBins && workers % 8 == 0 && (workers / 8) % kv_heads == 0;
   const int n_others = s_entries - 2 * n_pairs;
   // (when all of them are equally long there is nothing to even out: they go round the bins)
-  const int one_by_one = regular && s_sizes > 1 ? min(n_others, kDealtOneByOne) : 0;
+  const int candidates = regular && s_sizes > 1 ? min(n_others, kDealtOneByOne) : 0;
   auto bin_of_place = [&](int round, int x) { return (round & 1) ? per_round - 1 - x : x; };
   const int max_rounds = regular ? max((max_entries - batch) / per_round, 1) : 0;  // up to `batch` merge entries follow the places
+  int one_by_one = 0;  // entries dealt one by one (decided below)
   if (regular) {
     for (int x = tid; x < per_round; x += blockDim.x) {
       s_bin_load[x] = 0;
       s_bin_rounds[x] = 0;
+      s_snake_load[x] = 0;
     }
+    if (tid == 0) s_snake_max = s_snake_sum = 0;
     __syncthreads();
     // tiles of the entries by rank (a key is a tile count; ranks go down the keys), pairs' loads and rounds
-    for (int rank = tid; rank < n_pairs + one_by_one; rank += blockDim.x) {
+    for (int rank = tid; rank < n_pairs + candidates; rank += blockDim.x) {
       int lo = 0, hi = kKeys - 1;  // the smallest key whose entries start at or before this rank
       while (lo < hi) {
         const int mid = (lo + hi) >> 1;
@@ -340,8 +345,11 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
         atomicAdd(&s_bin_load[bin_of_place(round, x + half)], tiles);
         atomicMax(&s_bin_rounds[bin_of_place(round, x)], round + 1);
         atomicMax(&s_bin_rounds[bin_of_place(round, x + half)], round + 1);
-      } else if (rank - n_pairs < one_by_one) {
-        s_rank_tiles[rank - n_pairs] = tiles;
+      } else {
+        // (and what the plain snake deal - entry i to bin i, 2E-1-i, 2E+i, ... - would give each bin)
+        const int i = rank - n_pairs, lap = i / per_round;
+        s_rank_tiles[i] = tiles;
+        atomicAdd(&s_snake_load[(lap & 1) ? per_round - 1 - i % per_round : i % per_round], tiles);
       }
     }
     __syncthreads();
@@ -349,6 +357,19 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     if (pairing && n_pairs > 0)
       for (int x = tid; x < per_round; x += blockDim.x) s_bin_rounds[x] = max(s_bin_rounds[x], n_pairs / half);
     __syncthreads();
+    // Is the one-by-one deal worth its time (0.12 us an entry)?  If the heaviest
+    // bin of the plain snake deal over the sorted list is within 1/32 of the mean
+    // (batches of similar lengths), the snake it is.
+    if (candidates > 0) {
+      for (int x = tid; x < per_round; x += blockDim.x) {
+        const int load = s_bin_load[x] + s_snake_load[x];
+        atomicMax(&s_snake_max, load);
+        atomicAdd(&s_snake_sum, load);
+      }
+      __syncthreads();
+    }
+    const bool uneven = candidates > 0 && static_cast<long long>(s_snake_max) * per_round * 32 > static_cast<long long>(s_snake_sum) * 33;
+    one_by_one = uneven ? candidates : 0;
     // Entries beyond the first kDealtOneByOne (only large batches have them, and
     // they are the short ones) go round the bins in snake order, each into its
     // bin's next free round.
