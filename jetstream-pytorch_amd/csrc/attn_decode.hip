@@ -147,7 +147,7 @@ __device__ __forceinline__ unsigned wave_min_u32(unsigned x) {
 // access and no branch (an entry costs about a quarter of a microsecond less
 // than with LDS in the loop, and there are hundreds).
 template <int PER_LANE>
-__device__ __forceinline__ void deal_longest_first(int n, int per_round, int max_rounds, int* bin_load,
+__device__ __forceinline__ void deal_longest_first(int first, int n, int per_round, int max_rounds, int* bin_load,
                                                    int* bin_rounds, const int* rank_tiles, int* rank_place) {
   const int lane = threadIdx.x;
   unsigned mine[PER_LANE];
@@ -159,7 +159,7 @@ __device__ __forceinline__ void deal_longest_first(int n, int per_round, int max
     // a bin with no free round is out of the running (there is room for all: max_rounds * per_round)
     mine[i] = rounds[i] < max_rounds ? (static_cast<unsigned>(bin_load[x]) << 10) | static_cast<unsigned>(x) : ~0u;
   }
-  for (int block = 0; block < n; block += 64) {
+  for (int block = first; block < n; block += 64) {
     const int my_tiles = block + lane < n ? rank_tiles[block + lane] : 0;
     int my_place = 0;
     const int in_block = min(64, n - block);
@@ -196,6 +196,66 @@ __device__ __forceinline__ void deal_longest_first(int n, int per_round, int max
       bin_load[x] = static_cast<int>(mine[i] >> 10);  // a full bin reads as the heaviest, which suits what follows
     }
   }
+}
+
+// The same deal, many entries a step (at most 64 bins, one a lane).  The bins are
+// sorted by (tiles, bin) across the wave; entry i + j goes to the j-th lightest bin
+// for as long as that bin is lighter than every bin already given an entry of this
+// step is afterwards - exactly the choices of the one-by-one deal, which picks bin
+// j for entry i + j if and only if bin j's key is below the new keys of bins
+// 0..j-1.  Entries come in levels (every bin gets one of the long entries before
+// any gets a second), so a step usually places dozens: a sort of 21 exchanges and
+// a running minimum instead of a minimum per entry.  When a step places fewer than
+// eight (short entries on uneven bins), the rest is dealt one by one.  Returns the
+// first rank that is still to be dealt.
+__device__ __forceinline__ unsigned plan_sort_wave(unsigned key, int lane) {
+#pragma unroll
+  for (int k = 2; k <= 64; k <<= 1) {
+#pragma unroll
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      const unsigned other = static_cast<unsigned>(__shfl_xor(static_cast<int>(key), j));
+      const bool up = (lane & k) == 0, lower = (lane & j) == 0;
+      key = (lower == up) ? min(key, other) : max(key, other);
+    }
+  }
+  return key;
+}
+__device__ __forceinline__ int deal_longest_first_in_steps(int n, int per_round, int max_rounds, int* bin_load,
+                                                           int* bin_rounds, const int* rank_tiles, int* rank_place) {
+  const int lane = threadIdx.x;
+  int first = 0;
+  while (first < n) {
+    unsigned key = ~0u;  // a bin with no free round is out of the running
+    if (lane < per_round && bin_rounds[lane] < max_rounds) key = (static_cast<unsigned>(bin_load[lane]) << 10) | static_cast<unsigned>(lane);
+    key = plan_sort_wave(key, lane);
+    const bool has_entry = first + lane < n && key != ~0u;
+    const unsigned tiles = has_entry ? static_cast<unsigned>(rank_tiles[first + lane]) : 0u;
+    const unsigned after = has_entry ? key + (tiles << 10) : ~0u;
+    // the lightest of the bins before this lane once they have their entries (exclusive running minimum)
+    unsigned before = after;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const unsigned y = static_cast<unsigned>(__shfl_up(static_cast<int>(before), off));
+      if (lane >= off) before = min(before, y);
+    }
+    before = static_cast<unsigned>(__shfl_up(static_cast<int>(before), 1));
+    if (lane == 0) before = ~0u;
+    const bool ok = has_entry && key < before;
+    const unsigned long long bad = ~__ballot(ok);  // lanes whose entry is not this step's
+    const int placed = bad == 0 ? 64 : __ffsll(static_cast<long long>(bad)) - 1;
+    if (lane < placed) {
+      const int x = static_cast<int>(key & 1023u);
+      const int round = bin_rounds[x];
+      rank_place[first + lane] = round * per_round + ((round & 1) ? per_round - 1 - x : x);
+      bin_rounds[x] = round + 1;
+      bin_load[x] = static_cast<int>(key >> 10) + static_cast<int>(tiles);
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    first += placed;
+    if (placed < 8) break;
+  }
+  return first;
 }
 
 __global__ void __launch_bounds__(256)
@@ -376,9 +436,14 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     const int laps_after = (n_others - one_by_one + per_round - 1) / per_round;
     if (tid < 64 && one_by_one > 0) {
       const int cap = max(max_rounds - laps_after, 1);
-      if (per_round <= 64) deal_longest_first<1>(one_by_one, per_round, cap, s_bin_load, s_bin_rounds, s_rank_tiles, s_rank_place);
-      else if (per_round <= 256) deal_longest_first<4>(one_by_one, per_round, cap, s_bin_load, s_bin_rounds, s_rank_tiles, s_rank_place);
-      else deal_longest_first<16>(one_by_one, per_round, cap, s_bin_load, s_bin_rounds, s_rank_tiles, s_rank_place);
+      if (per_round <= 64) {
+        const int dealt = deal_longest_first_in_steps(one_by_one, per_round, cap, s_bin_load, s_bin_rounds, s_rank_tiles, s_rank_place);
+        deal_longest_first<1>(dealt, one_by_one, per_round, cap, s_bin_load, s_bin_rounds, s_rank_tiles, s_rank_place);
+      } else if (per_round <= 256) {
+        deal_longest_first<4>(0, one_by_one, per_round, cap, s_bin_load, s_bin_rounds, s_rank_tiles, s_rank_place);
+      } else {
+        deal_longest_first<16>(0, one_by_one, per_round, cap, s_bin_load, s_bin_rounds, s_rank_tiles, s_rank_place);
+      }
     }
     __syncthreads();
   }

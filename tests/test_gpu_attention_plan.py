@@ -5,6 +5,10 @@ lengths, the work entries cover every position of every slot exactly once;
 the two chunks of a slot cut in two sit on places that one workgroup's two
 groups walk in the same round, with every earlier round full; every other cut
 slot has consecutive partial records and one merge entry that names them all.
+The deal itself is pinned too: a host model of the planner's rule - entries that
+are not a pair's go, longest first, to the bin with the fewest tiles so far (or
+round the bins in snake order when that is even enough already) - must put the
+same number of tiles on every place as the plan read back from the device.
 """
 import numpy as np
 import pytest
@@ -31,6 +35,57 @@ def read_plan(plan):
   n_places, n_merges = int(state[2]), int(state[3])
   entries = raw[STATE_BYTES:STATE_BYTES + (n_places + n_merges) * ENTRY_INTS * 4].view(np.int32).reshape(-1, ENTRY_INTS)
   return entries[:n_places], entries[n_places:]
+
+
+DEALT_ONE_BY_ONE = 512  # entries the planner deals to the lightest bin; later ones go round the bins
+
+
+def model_deal(places, batch, kv_heads):
+  """Tiles the planner's rule puts on every place (-1: nobody), from the plan's own
+  entries: pairs stay where they are; the other entries, in sort order (chunks of
+  slots cut in three or more before whole slots, each longest first), are dealt
+  as plan_kernel deals them."""
+  w = workers()
+  per_round, half = w // kv_heads, w // kv_heads // 2
+  tiles_of = lambda count: min((count + TILE - 1) // TILE, 256)
+  is_pair = lambda e: e[0] >= 0 and e[3] == -1 and e[4] == 2
+  bin_of = lambda rnd, x: per_round - 1 - x if rnd & 1 else x
+  load, rounds = [0] * per_round, [0] * per_round
+  out = [-1] * len(places)
+  n_pairs = 0
+  for at, e in enumerate(places):
+    if is_pair(e):
+      rnd, x = divmod(at, per_round)
+      first = e if x < half else places[at - half]  # both bins are charged the first chunk's tiles
+      load[bin_of(rnd, x)] += tiles_of(first[2])
+      rounds[bin_of(rnd, x)] = max(rounds[bin_of(rnd, x)], rnd + 1)
+      out[at] = tiles_of(e[2])
+      n_pairs += x < half
+  if n_pairs:
+    rounds = [max(r, n_pairs // half) for r in rounds]
+  others = sorted(((1 if e[4] > 1 else 0, tiles_of(e[2])) for e in places if e[0] >= 0 and not is_pair(e)), reverse=True)
+  candidates = min(len(others), DEALT_ONE_BY_ONE) if len(set(others)) > 1 else 0
+  snake = list(load)
+  for i in range(candidates):
+    lap, x = divmod(i, per_round)
+    snake[per_round - 1 - x if lap & 1 else x] += others[i][1]
+  one_by_one = candidates if candidates and max(snake) * per_round * 32 > sum(snake) * 33 else 0
+  target = w * 5 // 4
+  extra = (target + kv_heads - 1) // kv_heads + 1
+  max_entries = (2 * batch + 2 * extra + 3 * (w // kv_heads + 8) + 7) // 8 * 8
+  max_rounds = max((max_entries - batch) // per_round, 1)
+  cap = max(max_rounds - (len(others) - one_by_one + per_round - 1) // per_round, 1)
+  for _, t in others[:one_by_one]:
+    x = min((b for b in range(per_round) if rounds[b] < cap), key=lambda b: (load[b], b))
+    out[rounds[x] * per_round + bin_of(rounds[x], x)] = t
+    load[x] += t
+    rounds[x] += 1
+  for i, (_, t) in enumerate(others[one_by_one:]):
+    lap, x = divmod(i, per_round)
+    x = per_round - 1 - x if lap & 1 else x
+    rnd = rounds[x] + lap
+    out[rnd * per_round + bin_of(rnd, x)] = t
+  return out
 
 
 def check_plan(lengths, kv_heads, seq):
@@ -82,6 +137,9 @@ def check_plan(lengths, kv_heads, seq):
     assert not used_parts & set(range(part0, part0 + n))
     used_parts |= set(range(part0, part0 + n))
   assert len(merge_of) == sum(1 for s in range(batch) if len(chunks[s]) > 1) - n_pairs
+  if 1 <= per_round <= 1024 and workers() % 8 == 0 and (workers() // 8) % kv_heads == 0:
+    got = [min((int(e[2]) + TILE - 1) // TILE, 256) if e[0] >= 0 else -1 for e in places]
+    assert got == model_deal([[int(v) for v in e] for e in places], batch, kv_heads), "the deal is not the model's"
   return n_pairs, len(merge_of)
 
 
@@ -107,6 +165,11 @@ def test_plan_covers_every_position_once_lognormal(seed):
     ([2048] * 40, 8, 2048),             # more pairs than one round holds
     ([1024] * 4096, 2, 1024),           # the largest batch the planner takes
     ([700] * 5, 3, 1024),               # a head count the workers do not divide by: no pairing
+    ([0] * 100 + [3000, 17, 900], 8, 4096),          # many entries of no tiles: one bin takes them all
+    (list(range(1, 2048, 7)), 8, 2048),               # evenly spread lengths
+    ([16] * 300 + [4000] * 30 + [100] * 90, 8, 4096), # short entries on uneven bins: few a step, then one by one
+    (list(range(5, 1500, 11)), 16, 2048),             # 32 bins
+    (list(range(5, 900, 3)), 4, 1024),                # 128 bins: two a lane
 ])
 def test_plan_covers_every_position_once_edge_cases(lengths, kv_heads, seq):
   check_plan(lengths, kv_heads, seq)
