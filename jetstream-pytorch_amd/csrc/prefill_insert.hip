@@ -293,6 +293,107 @@ __device__ __forceinline__ void quant_insert_tokens(const jpt_prefill_insert_arg
   }
 }
 
+// The same for the Llama shape, 8 heads of 128 elements, laid out for memory: a
+// thread keeps one 16-byte piece of one token's row in four heads (passes), so
+// that the 64 lanes of a wave read four consecutive tokens' rows of one head -
+// 1 KiB in one piece - and write 512 contiguous bytes of codes, where the
+// mapping above touches four heads' 256 bytes.  A token's absmax: over the
+// thread's four heads, the 16 lanes that share the token, and (one scale a
+// token) the workgroup's other half, which has the other four heads.
+template <bool BF16_MATH>
+__device__ __forceinline__ void quant_insert_tokens_8x128(const jpt_prefill_insert_args& a, const uint16_t* src, char* dst,
+                                                          void* scale_out, int t0) {
+  constexpr int H = 8, D = 128, kHeadsPerThread = 4;
+  const int piece = threadIdx.x & 15, tq = (threadIdx.x >> 4) & 7, hg = threadIdx.x >> 7;
+  const bool paged = a.page_ids != nullptr;
+  const int rows = paged ? a.n_pages * a.page_size : a.tokens;
+  const int groups = a.scale_heads;
+  const int64_t head_stride = a.src_head_stride > 0 ? a.src_head_stride : static_cast<int64_t>(a.tokens) * D;
+  const int t = t0 + tq, d = 8 * piece;
+  const int t_src = min(t, a.tokens - 1);
+  uint4 raw[kHeadsPerThread];
+#pragma unroll
+  for (int j = 0; j < kHeadsPerThread; ++j) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 w = __builtin_nontemporal_load(
+        reinterpret_cast<const u32x4*>(src + (hg * kHeadsPerThread + j) * head_stride + static_cast<int64_t>(t_src) * D + d));
+    raw[j] = make_uint4(w.x, w.y, w.z, w.w);
+  }
+  const int page = paged ? a.page_ids[min(t, rows - 1) / a.page_size] : 0;
+  int64_t pool_row = -1;  // dense: position in the slot's row; paged: row in the pool; -1: nothing to write
+  if (t < rows) {
+    if (paged) {
+      if (page >= 0 && page < a.total_pages) pool_row = static_cast<int64_t>(page) * a.page_size + t % a.page_size;
+    } else {
+      const int at = (a.start + t) % a.seq;
+      pool_row = at < 0 ? at + a.seq : at;
+    }
+  }
+  const bool live = t < a.tokens;
+  float x[kHeadsPerThread][8], m[kHeadsPerThread];
+#pragma unroll
+  for (int j = 0; j < kHeadsPerThread; ++j) {
+    const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+    m[j] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[j][2 * i] = live ? __uint_as_float(w[i] << 16) : 0.f;
+      x[j][2 * i + 1] = live ? __uint_as_float(w[i] & 0xffff0000u) : 0.f;
+      m[j] = fmaxf(m[j], fmaxf(fabsf(x[j][2 * i]), fabsf(x[j][2 * i + 1])));
+    }
+    for (int off = 8; off > 0; off >>= 1) m[j] = fmaxf(m[j], __shfl_xor(m[j], off));  // the head's 16 pieces
+  }
+  __shared__ float s_half[2][kTokensPerBlock];
+  if (groups == 1) {
+    const float mine = fmaxf(fmaxf(m[0], m[1]), fmaxf(m[2], m[3]));
+    if (piece == 0) s_half[hg][tq] = mine;
+    __syncthreads();
+    const float all = fmaxf(s_half[0][tq], s_half[1][tq]);
+#pragma unroll
+    for (int j = 0; j < kHeadsPerThread; ++j) m[j] = all;
+  }
+  if (pool_row < 0) return;
+#pragma unroll
+  for (int j = 0; j < kHeadsPerThread; ++j) {
+    const int h = hg * kHeadsPerThread + j;
+    const int64_t row = paged ? static_cast<int64_t>(h) * a.total_pages * a.page_size + pool_row
+                              : (static_cast<int64_t>(a.slot) * H + h) * a.seq + pool_row;
+    uint2* out = reinterpret_cast<uint2*>(dst + row * D + d);
+    if (!live) {  // paged only: the tail of the last page is zero-filled
+      *out = make_uint2(0u, 0u);
+      continue;
+    }
+    float amax = m[j];
+    if (a.rounding == JPT_ROUND_RNE) amax = fmaxf(amax, rnd<BF16_MATH>(1e-5f));
+    const float s = rnd<BF16_MATH>(amax / 127.0f);
+    uint32_t code[8];
+    if (a.rounding == JPT_ROUND_TRUNC) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float q = rnd<BF16_MATH>(x[j][i] / s);
+        code[i] = static_cast<uint32_t>((q != q) ? 0 : static_cast<int>(q)) & 0xffu;
+      }
+    } else {
+      const float r = rnd<BF16_MATH>(1.0f / s);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float q = rnd<BF16_MATH>(x[j][i] * r);
+        code[i] = static_cast<uint32_t>(static_cast<int>(fminf(fmaxf(rintf(q), -128.f), 127.f))) & 0xffu;
+      }
+    }
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 packed = {code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24),
+                          code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24)};
+    __builtin_nontemporal_store(packed, reinterpret_cast<u32x2*>(out));
+    if (piece == 0 && (groups == 1 ? (hg == 0 && j == 0) : true)) {
+      const int g = groups == 1 ? 0 : h;
+      const int64_t idx = paged ? static_cast<int64_t>(g) * a.total_pages * a.page_size + pool_row
+                                : (static_cast<int64_t>(a.slot) * groups + g) * a.seq + pool_row;
+      store_from_f32(scale_out, idx, a.scale_dtype, s);
+    }
+  }
+}
+
 template <bool BF16_MATH>
 __global__ void __launch_bounds__(256) prefill_insert_quant4_kernel(InsertParams p) {
   const jpt_prefill_insert_args& a = p.a;
@@ -301,7 +402,10 @@ __global__ void __launch_bounds__(256) prefill_insert_quant4_kernel(InsertParams
   char* dst;
   void* scale_out;
   layer_tensors(p, blockIdx.z, is_v, 2, 1, a.scale_dtype == JPT_F32 ? 4 : 2, &src, &dst, &scale_out);
-  quant_insert_tokens<BF16_MATH>(a, static_cast<const uint16_t*>(src), dst, scale_out, blockIdx.x * kTokensPerBlock);
+  if (a.heads == 8 && a.dim == 128)
+    quant_insert_tokens_8x128<BF16_MATH>(a, static_cast<const uint16_t*>(src), dst, scale_out, blockIdx.x * kTokensPerBlock);
+  else
+    quant_insert_tokens<BF16_MATH>(a, static_cast<const uint16_t*>(src), dst, scale_out, blockIdx.x * kTokensPerBlock);
 }
 
 // Several prompts into the pages of one stacked pool in one launch: the
@@ -331,7 +435,9 @@ __global__ void __launch_bounds__(256) prefill_insert_prompts_kernel(PromptsPara
   char* dst = static_cast<char*>(is_v ? a.dst_v : a.dst_k) + layer * a.dst_layer_stride;
   const int esz_scale = a.scale_dtype == JPT_F32 ? 4 : 2;
   void* scale_out = static_cast<char*>(is_v ? a.v_scale : a.k_scale) + layer * a.scale_layer_stride * esz_scale;
-  quant_insert_tokens<BF16_MATH>(a, src, dst, scale_out, (static_cast<int>(blockIdx.x) - p.first_block[r]) * kTokensPerBlock);
+  const int t0 = (static_cast<int>(blockIdx.x) - p.first_block[r]) * kTokensPerBlock;
+  if (a.heads == 8 && a.dim == 128) quant_insert_tokens_8x128<BF16_MATH>(a, src, dst, scale_out, t0);
+  else quant_insert_tokens<BF16_MATH>(a, src, dst, scale_out, t0);
 }
 
 }  // namespace
