@@ -335,12 +335,25 @@ int32_t jpt_prefill_insert_prompts(const jpt_prefill_insert_args* args,
  * (JPT_E_BADARG; the reference raises on them, attention_kernel.py:525-526,
  * :547-550).  Every wait inside the streaming kernel is bounded; a wave whose
  * wait runs out gives up, the launch ends, and word 0 of the state block is
- * set and stays set: what the launch wrote is then not to be used.  The launch
- * itself cannot report this (the call only enqueues); jpt_attn_status does.
+ * set and stays set: what the launch wrote - and what every later launch on
+ * that workspace writes until jpt_attn_status has been called - is then not to
+ * be used.  The launch itself cannot report this (the call only enqueues);
+ * jpt_attn_status does, and puts the workspace's counters back to what a
+ * fresh plan holds, so the plan stays usable afterwards.
+ *
+ * The device must be the launch's own.  The streaming kernel is one
+ * persistent workgroup per compute unit (all of a unit's LDS), and a slot
+ * that is cut into three or more chunks is folded by a wave that waits -
+ * up to a tenth of a second - for chunks that belong to OTHER workgroups of
+ * the same launch.  If part of the grid cannot be resident while the rest
+ * runs (compute units masked off, or held for that long by a kernel of another
+ * stream or process), that wait runs out and the launch gives up.  Kernels of
+ * other streams that merely share the device delay it, they do not break it.
  * ---------------------------------------------------------------------- */
 #define JPT_ATTN_WS_STATE_BYTES 65536
 #define JPT_ATTN_STATUS_GAVE_UP 1
 #define JPT_ATTN_STATUS_SLOT_FULL 2
+#define JPT_ATTN_STATUS_PLAN_OVERFLOW 4
 
 typedef struct {
   const void* q;
@@ -418,11 +431,17 @@ int32_t jpt_attn_ragged_static(const jpt_attn_args* args, void* stream);
  * and clears it.  Bits, sticky since the last call:
  *   JPT_ATTN_STATUS_GAVE_UP    a launch gave up (see Errors above);
  *   JPT_ATTN_STATUS_SLOT_FULL  a plan saw a slot whose length had reached the
- *     cache capacity (seq, or max_pages * page_size): the slot is attended up
- *     to the capacity, and a token appended to it in that step is attended
- *     but NOT stored (every append on this path skips positions outside the
- *     cache; the reference's dynamic_update_slice would clamp the position
- *     and overwrite the last row, cache_manager.py:154-173).
+ *     cache capacity (seq, or max_pages * page_size), whether or not the step
+ *     carries a token: the slot is attended up to the capacity, and a token
+ *     appended to it in that step is attended but NOT stored (every append on
+ *     this path skips positions outside the cache; the reference's
+ *     dynamic_update_slice would clamp the position and overwrite the last
+ *     row, cache_manager.py:154-173);
+ *   JPT_ATTN_STATUS_PLAN_OVERFLOW  a plan had more entries than its array
+ *     holds (a fault of the library's own accounting): positions were left
+ *     out, the results of launches on that plan are not to be used.
+ * After JPT_ATTN_STATUS_GAVE_UP the call also clears the plan's arrival and
+ * hand-out counters, which the launch that gave up may have left half counted.
  *  Synchronises: call it where the caller synchronises anyway (the
  * reference raises from inside its jitted step; a kernel cannot).  Not to be
  * called during stream capture.  workspace NULL: the library's own workspace

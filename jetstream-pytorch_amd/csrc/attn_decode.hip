@@ -261,6 +261,9 @@ __device__ __forceinline__ int deal_longest_first_in_steps(int n, int per_round,
 __global__ void __launch_bounds__(256)
 plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int target, int workers,
             PlanEntry* entries, int32_t* arrivals, int max_entries, int32_t* status) {
+  // An entry that does not fit the plan's array would be positions nobody attends: the capacity
+  // (make_layout) is sized so that this cannot happen, and if it ever does the launch says so.
+  auto overflow = [&]() { atomicOr(status, JPT_ATTN_STATUS_PLAN_OVERFLOW); };
   constexpr int kKeys = 3 * 257;  // tile count; + 257: chunks of slots cut in three or more; + 514: in two, paired
   __shared__ int s_len[kMaxPlanBatch];
   __shared__ int s_first[kMaxPlanBatch];
@@ -465,6 +468,8 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
         entries[at] = PlanEntry{b, 0, cl, -1, 2, s_len[b], {0, 0}};
         entries[at + half] = PlanEntry{b, cl, s_len[b] - cl, -1, 2, s_len[b], {0, 0}};
         atomicMax(&s_positions, at + half + 1);
+      } else {
+        overflow();
       }
       continue;
     }
@@ -474,6 +479,8 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
       if (at < max_entries) {
         entries[at] = PlanEntry{b, c * cl, count, first + c, nc, s_len[b], {0, 0}};
         atomicMax(&s_positions, at + 1);
+      } else {
+        overflow();
       }
     }
   }
@@ -485,12 +492,15 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     if (nc > 1 && !paired(b)) {
       const int at = n_places + atomicAdd(&s_merges, 1);
       if (at < max_entries) entries[at] = PlanEntry{b, -1, 0, s_first[b], nc, s_len[b], {0, 0}};
+      else overflow();
     }
   }
   __syncthreads();
   if (tid < kHandOutCounters) status[kStateHandOut + tid * kStateHandOutStride] = 0;
   if (tid == 0) {
     status[kStateEntries] = n_places;
+    status[kStateArrivalsAt] = static_cast<int32_t>(arrivals - status);
+    status[kStateArrivalsCount] = batch * kv_heads;
     status[kStateMerges] = max(min(n_places + s_merges, max_entries) - n_places, 0);
   }
 }
@@ -691,11 +701,22 @@ int32_t jpt_attn_status(void* workspace, void* stream, int32_t* status) {
     if (workspace == nullptr) return st;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  int32_t word = 0;
-  JPT_HIP(hipMemcpyAsync(&word, workspace, sizeof(word), hipMemcpyDeviceToHost, s));
+  // words 0 .. kStateArrivalsCount of the state block
+  int32_t head[kStateArrivalsCount + 1] = {0};
+  JPT_HIP(hipMemcpyAsync(head, workspace, sizeof(head), hipMemcpyDeviceToHost, s));
   JPT_HIP(hipStreamSynchronize(s));
+  const int32_t word = head[kStateStatus];
   if (word != 0) {
     JPT_HIP(hipMemsetAsync(workspace, 0, sizeof(word), s));
+    if (word & JPT_ATTN_STATUS_GAVE_UP) {
+      // The launch that gave up may have left arrival counts behind, and chunks counted
+      // without their merge; a launch reusing the plan would take them for this launch's.
+      // Back to what a fresh plan holds.
+      int32_t* ws = static_cast<int32_t*>(workspace);
+      JPT_HIP(hipMemsetAsync(ws + kStateHandOut, 0, kHandOutCounters * kStateHandOutStride * sizeof(int32_t), s));
+      if (head[kStateArrivalsAt] > 0 && head[kStateArrivalsCount] > 0)
+        JPT_HIP(hipMemsetAsync(ws + head[kStateArrivalsAt], 0, static_cast<size_t>(head[kStateArrivalsCount]) * sizeof(int32_t), s));
+    }
     JPT_HIP(hipStreamSynchronize(s));
   }
   *status = word;

@@ -68,6 +68,7 @@ constexpr int kSideBytes = 512;     // ks | vs | mask, 128 bytes each at most
 constexpr int kOStride = 140;       // padded LDS row of 128 outputs
 constexpr int kLdsBudget = 160 * 1024 / kGroups - 512;  // per group; one workgroup per compute unit
 constexpr int kSpinLimit = 1 << 18;  // tens of milliseconds
+constexpr uint64_t kMergeWaitTicks = 10 * 1000 * 1000;  // 0.1 s of the 100 MHz clock: a merge's wait for other workgroups' chunks
 // Cache policy of the loads that stream the cache (keys, values, their scales):
 // non-temporal - every byte is read once per launch, and lines kept for it in
 // the caches only push out what is read again (query rows, page ids, masks).
@@ -593,11 +594,16 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
   // folds the partials and writes the slot's output.  One wave's work.
   auto merge_item = [&](const Item& it) -> bool {
     int32_t* counter = p.arrivals + static_cast<int64_t>(it.slot) * a.kv_heads + it.h;
-    for (int spins = 0;; ++spins) {
+    // The chunks belong to other workgroups, which must get to run for this wait
+    // to end: it is sized in time (the constant 100 MHz clock), long enough for
+    // workgroups held back by other work on the device to be scheduled.
+    const uint64_t wait_from = __builtin_amdgcn_s_memrealtime();
+    for (;;) {
       int seen = 0;
       if (lane == 0) seen = __hip_atomic_fetch_add(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (__builtin_amdgcn_readfirstlane(seen) >= it.n_chunks) break;
-      if (spins > (kSpinLimit >> 6) || __hip_atomic_load(&sm_abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) {
+      if (__builtin_amdgcn_s_memrealtime() - wait_from > kMergeWaitTicks ||
+          __hip_atomic_load(&sm_abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) {
         give_up();
         return false;
       }
@@ -977,21 +983,26 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
     // that are done first do the merging, which costs the launch no tail.  The
     // workers of workgroups equal mod 8 share one counter and the pairs equal to
     // them mod 8 (a dozen nanoseconds per atomic add on one address: one counter
-    // for everybody would queue).  Every worker asks until it is refused once, so
-    // a launch advances a counter by exactly its pairs plus its workers, and
-    // launches that follow one another on a plan need no reset: the counter's
-    // value modulo that sum is the place in the current launch.
+    // for everybody would queue).  Every worker asks until it is refused once:
+    // a launch asks a counter exactly pairs + workers times, and the counter
+    // counts modulo that number (a wrapping increment), so it is back where it
+    // started when the launch ends, launches that follow one another on a plan
+    // need no reset, and the counter never grows.  Whatever value a launch finds
+    // in it - one that an aborted launch left behind, say - every merge place is
+    // handed out exactly once: the asks walk the whole cycle from wherever it
+    // starts, and a value outside the cycle costs the first asker a refusal and
+    // puts the counter back to zero.
     const int n_merges = load_uniform(p.status + kStateMerges);
     const int share = worker & 7;
     const int sharers = (G - share + 7) / 8;
     const int pairs = n_merges * a.kv_heads;
     const int my_pairs = pairs > share ? (pairs - share + 7) / 8 : 0;
     const unsigned per_launch = static_cast<unsigned>(my_pairs + sharers);
-    int32_t* const hand_out = p.status + kStateHandOut + share * kStateHandOutStride;
+    unsigned* const hand_out = reinterpret_cast<unsigned*>(p.status + kStateHandOut + share * kStateHandOutStride);
     for (;;) {
-      int number = 0;
-      if (lane == 0) number = __hip_atomic_fetch_add(hand_out, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const unsigned place = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(number)) % per_launch;
+      unsigned number = 0;
+      if (lane == 0) number = __builtin_amdgcn_atomic_inc32(hand_out, per_launch - 1, __ATOMIC_RELAXED, "agent");
+      const unsigned place = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(number)));
       if (place >= static_cast<unsigned>(my_pairs)) break;
       const int pair = share + 8 * static_cast<int>(place);
       const int32_t* en = reinterpret_cast<const int32_t*>(p.entries + n_entries + pair / a.kv_heads);

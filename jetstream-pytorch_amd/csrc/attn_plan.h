@@ -25,6 +25,10 @@ struct PlanEntry {
 constexpr int kStateStatus = 0;    // sticky JPT_ATTN_STATUS_* bits
 constexpr int kStateEntries = 2;   // plan entries that are work items (chunks and whole slots)
 constexpr int kStateMerges = 3;    // merge entries, which follow them
+// where the plan's arrival counters lie (32-bit words from the workspace's start) and how many
+// there are: what jpt_attn_status clears, with the hand-out counters, after a launch gave up
+constexpr int kStateArrivalsAt = 4;
+constexpr int kStateArrivalsCount = 5;
 // merge entries handed out, one counter for the workers of workgroups equal mod 8
 // (one XCD), each in a cache line of its own (see the streaming kernel)
 constexpr int kStateHandOut = 16;

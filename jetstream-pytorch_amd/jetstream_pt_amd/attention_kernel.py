@@ -68,17 +68,23 @@ def _streaming_kernel_may_run(rows, dim, q_dtype, kv_dtype):
           and kv_dtype in (torch.int8, torch.bfloat16))
 
 
-STATUS_GAVE_UP, STATUS_SLOT_FULL = 1, 2
+STATUS_GAVE_UP, STATUS_SLOT_FULL, STATUS_PLAN_OVERFLOW = 1, 2, 4
 
 
 def check_status(plan=None):
   """Raises RuntimeError if a streaming-kernel launch gave up since the last
-  check (a bounded in-kernel wait ran out: its outputs are not to be used).
-  Looks at `plan`'s workspace, or at every workspace still alive (the shared
-  ones and those of every DecodePlan).
-  Synchronises the current stream; the record is cleared by the check.
+  check (a bounded in-kernel wait ran out: its outputs, and those of every
+  launch on that workspace since, are not to be used), or if a plan did not fit
+  its array.  Looks at `plan`'s workspace, or at every workspace still alive
+  (the shared ones and those of every DecodePlan).
+  Synchronises the current stream; the record is cleared by the check, and
+  after a launch that gave up the library puts the plan's counters back, so
+  the plan can be used again.  Call it where the decode loop synchronises
+  anyway - where the step's ResultTokens (engine.py:828-834) are copied to the
+  host - not inside a captured step.
   Returns the remaining status bits: STATUS_SLOT_FULL says that a planned step
-  saw a slot at cache capacity, whose new token was attended but not stored."""
+  saw a slot at cache capacity, whose new token (if the step carries one) was
+  attended but not stored."""
   if plan is not None:
     spaces = [plan.workspace]
   else:
@@ -91,7 +97,10 @@ def check_status(plan=None):
   if bad & STATUS_GAVE_UP:
     raise RuntimeError("a decode attention launch gave up on a bounded wait inside the kernel; "
                        "its outputs (and any token it was to quantise or append) are not valid")
-  return bad
+  if bad & STATUS_PLAN_OVERFLOW:
+    raise RuntimeError("a decode attention plan had more entries than its array holds; "
+                       "the outputs of launches on that plan are not valid")
+  return bad & ~(STATUS_GAVE_UP | STATUS_PLAN_OVERFLOW)
 
 
 def _shared_workspace(nbytes, device):

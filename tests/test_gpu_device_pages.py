@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 import torch
 
+from conftest import attention_bound
 from oracle import decode_state as ods
 from oracle.page_manager import PageAttentionManager as OPam
 
@@ -240,8 +241,9 @@ def test_paged_decode_steps_device_allocator_equals_host_allocator(int8, fused):
       assert torch.equal(got, want), what
       return
     live = torch.from_numpy(lens > 0).to(DEV)  # inactive slots: nothing is attended
+    # `want` is the separate launches' bf16 output: half an ulp of its own on top
     err = (got.float() - want.float()).abs()[live]
-    assert torch.all(err <= 1e-2 + 1e-2 * want.float().abs()[live]), f"{what}: max err {err.max():.4g}"
+    assert torch.all(err <= attention_bound(want.float(), rounded_want=True)[live]), f"{what}: max err {err.max():.4g}"
 
   def new_inputs():
     for t in (xq, xk, xv):

@@ -26,14 +26,10 @@ def _case(g, b, hq, hkv, s, lens):
   return q, k, v, ks, vs, xk, xv, end
 
 
-def _run(fn, case, workspace):
-  """One launch that quantises and attends the step's token too (every kind of
-  scratch use: plan, partials of split slots, status word).  Returns every
-  tensor the launch writes."""
-  from jetstream_pt_amd import _ffi
-  q, k, v, ks, vs, xk, xv, end = case
+def _outputs(case):
+  q, k = case[0], case[1]
   b, hq, _, d = q.shape
-  hkv, s = k.shape[1], k.shape[2]
+  hkv = k.shape[1]
   out = torch.empty_like(q)
   omax = torch.empty((b, hq, 1), dtype=torch.float32, device=DEV)
   oden = torch.empty_like(omax)
@@ -41,6 +37,18 @@ def _run(fn, case, workspace):
   nv = torch.empty_like(nk)
   nks = torch.empty((b, 1), dtype=torch.float32, device=DEV)
   nvs = torch.empty_like(nks)
+  return out, omax, oden, nk, nv, nks, nvs
+
+
+def _run(fn, case, workspace, outputs=None):
+  """One launch that quantises and attends the step's token too (every kind of
+  scratch use: plan, partials of split slots, status word).  Returns every
+  tensor the launch writes (`outputs`, or new ones)."""
+  from jetstream_pt_amd import _ffi
+  q, k, v, ks, vs, xk, xv, end = case
+  b, hq, _, d = q.shape
+  hkv, s = k.shape[1], k.shape[2]
+  out, omax, oden, nk, nv, nks, nvs = outputs if outputs is not None else _outputs(case)
   a = _ffi.AttnArgs(
       q=_ffi.ptr(q), k=_ffi.ptr(k), v=_ffi.ptr(v), k_scale=_ffi.ptr(ks), v_scale=_ffi.ptr(vs),
       lengths=_ffi.ptr(end), new_k=_ffi.ptr(nk), new_v=_ffi.ptr(nv), new_k_scale=_ffi.ptr(nks),
@@ -78,6 +86,17 @@ def test_static_scratch_entry_point_matches_and_allocates_nothing():
     outputs = sum(t.numel() * t.element_size() for t in got)
     assert torch.cuda.max_memory_allocated() - before <= outputs + 8 * 512  # torch rounds each tensor up
     for name, x, y in zip("out max denom new_k new_v new_k_scale new_v_scale".split(), got, want):
+      assert torch.equal(x, y), name
+    # torch's counters above see torch's allocator only.  The device's own: with the outputs
+    # allocated beforehand, a call (not the process's first, which loads what the runtime loads
+    # once) leaves the device's free memory exactly where it was.
+    outputs = _outputs(case)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    again = _run(_ffi.lib.jpt_attn_ragged_static, case, None, outputs)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "device memory was allocated or freed during the call"
+    for name, x, y in zip("out max denom new_k new_v new_k_scale new_v_scale".split(), again, want):
       assert torch.equal(x, y), name
     word = ctypes.c_int32(-1)
     _ffi.check(_ffi.lib.jpt_attn_status(None, _ffi.stream(), ctypes.byref(word)))
