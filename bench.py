@@ -24,9 +24,11 @@ by its time; `roofline` is the attention launch alone (a separate timed loop
 of attention launches only); `cpu_baseline` times the CPU oracle's
 restatement of the reference path on the host cores.
 
-The other configurations of BASELINE.json are parity-test cases; `--workload
-c1|c2|c4|c5` times them the same way for the record (same JSON shape, no
-cpu_baseline):
+The other configurations of BASELINE.json are parity-test cases; the default run
+times them after the headline, the same way, and adds them to the same JSON line
+as `other_workloads` (layer-step and attention launch of each; the headline
+fields stay C3's); `--workload c1|c2|c4|c5` times one of them alone (same JSON
+shape, no cpu_baseline):
   c1  dense bf16 eager update + dense attention, B=8, 32 heads, S=1024
   c2  int8 MHA decode step, B=96, 32 heads, S=2048, lengths U[128, 2048] (a slot at
       2048 is full: it is attended, its new token is attended too but not stored)
@@ -297,16 +299,49 @@ def build_paged(torch, args, int8):
   if int8:
     caches = [cm.Int8PageKVCacheGenerate(pools_k[l], pools_v[l], sk[l], sv[l], pam, None, env=env) for l in range(nl)]
     kernels = [layers.Int8KVAttentionKernel(env, l) for l in range(nl)]
-    prompt_k = torch.randn((nl, hkv, 1024, D), generator=gd, device=DEV).to(torch.bfloat16)
-    prompt_v = torch.randn((nl, hkv, 1024, D), generator=gd, device=DEV).to(torch.bfloat16)
+    # Every prompt of a decode step comes from a buffer of its own (16 x (K + V) x 64 MiB = 2 GiB a
+    # step at 32 layers), so that the insert reads HBM: slices of one buffer would sit in the
+    # 256 MB memory-side cache from the second prompt on.
+    prompt_k = torch.randn((16, nl, hkv, 1024, D), generator=gd, device=DEV).to(torch.bfloat16)
+    prompt_v = torch.randn((16, nl, hkv, 1024, D), generator=gd, device=DEV).to(torch.bfloat16)
   else:
     caches = [cm.PageKVCacheGenerate(pools_k[l], pools_v[l], pam, None, env=env) for l in range(nl)]
     kernels = [layers.AttentionKernel(env, l) for l in range(nl)]
-  state = {"lens": lengths.copy(), "decode_steps": 0, "attended": 0, "pages": 0, "inserted": 0, "log": []}
+  state = {"lens": lengths.copy(), "decode_steps": 0, "attended": 0, "pages": 0, "inserted": 0, "log": [],
+           "prompts_used": 0}
   churn = 16 if int8 else 0
 
-  def to_dev_async(a):
-    return torch.from_numpy(a).pin_memory().to(DEV, non_blocking=True)
+  # Requests of a decode step go to the device through pinned staging buffers that exist
+  # before the timed loop (allocating pinned memory waits for the device): row 0 the slots to
+  # free, row 1 their new lengths (0 for a slot that retires), as int32 for the allocator and as
+  # int64 for torch's index_copy_.  A ring of them, each with the event of its last upload, so
+  # that the host can run passes ahead of the device.
+  ring_n = 64
+  stage = stage_dev = None
+  if not host_alloc:
+    stage = [(torch.empty((2, batch), dtype=torch.int32).pin_memory(), torch.empty((batch,), dtype=torch.int64).pin_memory())
+             for _ in range(ring_n)]
+    stage_dev = [(torch.empty((2, batch), dtype=torch.int32, device=DEV), torch.empty((batch,), dtype=torch.int64, device=DEV))
+                 for _ in range(ring_n)]
+  uploaded = [None] * ring_n
+  passes_run = [0]
+
+  def upload(slots, new_lens):
+    """slots and their new lengths (numpy int32) -> device views (slots, lens, slots as int64)."""
+    j = passes_run[0] % ring_n
+    passes_run[0] += 1
+    if uploaded[j] is not None:
+      uploaded[j].synchronize()
+    n = len(slots)
+    (h32, h64), (d32, d64) = stage[j], stage_dev[j]
+    h32[0, :n] = torch.from_numpy(slots)
+    h32[1, :n] = torch.from_numpy(new_lens)
+    h64[:n] = h32[0, :n]
+    d32.copy_(h32, non_blocking=True)
+    d64.copy_(h64, non_blocking=True)
+    uploaded[j] = torch.cuda.Event()
+    uploaded[j].record()
+    return d32[0, :n], d32[1, :n], d64[:n]
 
   def before_pass():
     """What the engine does once per decode step before the layers run: new
@@ -314,40 +349,47 @@ def build_paged(torch, args, int8):
     step are reserved and the tables uploaded.  Also the byte accounting."""
     lens = state["lens"]
     full = np.nonzero(lens >= max_pages * ps)[0].astype(np.int32)
-    if len(full):  # a slot at max_cache_len cannot take another token: its request is over, the slot retires
-      if host_alloc:
-        for slot in full:
-          pam.free_pages_resource(int(slot))
-      else:
-        dfull = to_dev_async(full)
-        pam.free_pages_resource_many(dfull)
-        dlens.index_fill_(0, dfull.long(), 0)
-      if log_on:
-        state["log"].append(("free_many", full.copy()))
-      lens[full] = 0
+    # a slot at max_cache_len cannot take another token: its request is over, the slot retires
+    if len(full) and host_alloc:
+      for slot in full:
+        pam.free_pages_resource(int(slot))
+    if len(full) and host_alloc:
+      state["log"].append(("free_many", full.copy()))
+    lens[full] = 0
+    slots = ns = np.zeros((0,), dtype=np.int32)
     if churn:
       slots = rng.choice(batch, churn, replace=False).astype(np.int32)
       ns = np.array([int(rng.integers(64, 1025)) for _ in slots], dtype=np.int32)
-      if host_alloc:
-        for slot, n in zip(slots, ns):
-          pam.free_pages_resource(int(slot))
-          _, ids = pam.reserve_pages_insert(int(slot), int(n))
-          ids = np.array(ids, dtype=np.int32)
-          gins.insert_prefix_pages_int8_stacked(prompt_k[:, :, :n], prompt_v[:, :, :n], pools_k, pools_v, sk, sv, ids)
-          state["log"].append(("insert", int(slot), int(n), ids))
-      else:
-        dslots, dns = to_dev_async(slots), to_dev_async(ns)
-        pam.free_pages_resource_many(dslots)
-        pam.reserve_pages_insert_many(dslots, dns)
-        dlens.index_copy_(0, dslots.long(), dns)
-        # all of the step's prompts in one launch; page ids are views of the device table (no copy)
+    if host_alloc:
+      for slot, n in zip(slots, ns):
+        pam.free_pages_resource(int(slot))
+        _, ids = pam.reserve_pages_insert(int(slot), int(n))
+        ids = np.array(ids, dtype=np.int32)
+        j = state["prompts_used"] % 16
+        state["prompts_used"] += 1
+        gins.insert_prefix_pages_int8_stacked(prompt_k[j, :, :, :n], prompt_v[j, :, :, :n], pools_k, pools_v, sk, sv, ids)
+        state["log"].append(("insert", int(slot), int(n), ids, j))
+    elif len(full) or len(slots):
+      # one upload, one free (retired slots and the slots the new prompts take over), one
+      # reservation, one update of the engine's lengths, and all of the step's prompts in one
+      # insert launch; page ids are views of the device table (no copy)
+      retire = np.setdiff1d(full, slots).astype(np.int32)
+      dfree, dnew, dfree64 = upload(np.concatenate([retire, slots]), np.concatenate([np.zeros_like(retire), ns]))
+      pam.free_pages_resource_many(dfree)
+      if len(slots):
+        pam.reserve_pages_insert_many(dfree[len(retire):], dnew[len(retire):])
+      dlens.index_copy_(0, dfree64, dnew)
+      if len(slots):
         gins.insert_prompts_pages_int8_stacked(
-            [(prompt_k[:, :, :n], prompt_v[:, :, :n]) for n in ns], pools_k, pools_v, sk, sv,
+            [(prompt_k[j, :, :, :n], prompt_v[j, :, :, :n]) for j, n in enumerate(ns)], pools_k, pools_v, sk, sv,
             [pam.page_indices[int(slot), : (int(n) + ps - 1) // ps] for slot, n in zip(slots, ns)])
-        if log_on:
-          state["log"].append(("free_many", slots.copy()))
-          state["log"].append(("insert_many", slots.copy(), ns.copy(),
-                               [pam.page_indices[int(s), : (int(n) + ps - 1) // ps].cpu().numpy() for s, n in zip(slots, ns)]))
+      if log_on:
+        state["log"].append(("free_many", np.concatenate([retire, slots])))
+      if log_on and len(slots):
+        state["log"].append(("insert_many", slots.copy(), ns.copy(),
+                             [pam.page_indices[int(s), : (int(n) + ps - 1) // ps].cpu().numpy() for s, n in zip(slots, ns)],
+                             list(range(len(ns)))))
+    if len(slots):
       lens[slots] = ns
       state["inserted"] += int(ns.sum())
     if host_alloc:
@@ -576,6 +618,14 @@ def run_cpu_baseline(budget_s=20.0):
                      f"median of {len(times)} runs, {med * 1e3:.1f} ms each")
 
 
+T0 = time.perf_counter()
+
+
+def progress(what):
+  """A line on stderr per phase: a long run must show that it is alive."""
+  print(f"[bench {time.perf_counter() - T0:6.1f} s] {what}", file=sys.stderr, flush=True)
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -585,6 +635,8 @@ def main():
   ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c3")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   ap.add_argument("--no-graph", action="store_true", help="launch every step from Python")
+  ap.add_argument("--no-other-workloads", action="store_true",
+                  help="c3: skip the timing of c1, c2, c4 and c5 that follows the headline")
   ap.add_argument("--first-use-memory", action="store_true",
                   help="time the workload on its first allocation only (no free-and-allocate-again pass)")
   ap.add_argument("--host-alloc", action="store_true",
@@ -598,6 +650,7 @@ def main():
   if args.probe_traffic:
     run_traffic_probe(args)
     return
+  progress(f"{args.workload}: building and timing")
   r = run_gpu(args)
   first_use = None
   if not args.first_use_memory:
@@ -616,6 +669,7 @@ def main():
     del r
     gc.collect()
     torch.cuda.empty_cache()
+    progress(f"{args.workload}: built again on memory that has been used before")
     r = run_gpu(args)
   gbps = r["step_bytes"] / (r["ms_per_step"] * 1e-3) / 1e9
   attn_gbps = r["attn_bytes"] / (r["attn_ms"] * 1e-3) / 1e9
@@ -656,8 +710,41 @@ def main():
   if first_use is not None:
     cfg["memory"] = "synthetic cache allocated, freed and allocated again before timing; first_use_memory = the same run on the first allocation"
     line["first_use_memory"] = first_use
+  if headline and not args.no_other_workloads and not args.layers:
+    # The other four configurations of BASELINE.json, timed the same way in the same run, one
+    # after another (each is built, timed and freed before the next): for the record, the
+    # headline fields above are C3's alone.
+    import copy
+    import gc
+
+    import torch
+    del r
+    others = {}
+    for name in ("c1", "c2", "c4", "c5"):
+      gc.collect()
+      torch.cuda.empty_cache()
+      a2 = copy.copy(args)
+      a2.workload = name
+      progress(f"{name}: building and timing")
+      o = run_gpu(a2)
+      o_gbps = o["step_bytes"] / (o["ms_per_step"] * 1e-3) / 1e9
+      o_attn = o["attn_bytes"] / (o["attn_ms"] * 1e-3) / 1e9
+      others[name] = {
+          "workload": o["config"]["workload"], "layers_rotated": o["config"]["layers_rotated"],
+          "us_per_layer": round(o["ms_per_step"] * 1e3, 2), "min_us_per_layer": round(o["ms_min"] * 1e3, 2),
+          "mean_us_per_layer": round(o["ms_mean"] * 1e3, 2), "repeats": o["repeats"],
+          "GB_per_s": round(o_gbps, 1), "pct_of_hbm_peak": round(100 * o_gbps / HBM_PEAK_GBPS, 1),
+          "layer_step_bytes": int(o["step_bytes"]),
+          "attention": {"kernel": o["kernel"], "us_per_launch": round(o["attn_ms"] * 1e3, 2),
+                        "min_us_per_launch": round(o["attn_min"] * 1e3, 2), "GB_per_s": round(o_attn, 1),
+                        "frac": round(o_attn / HBM_PEAK_GBPS, 4), "algorithmic_bytes": int(o["attn_bytes"])},
+      }
+      del o
+    line["other_workloads"] = others
   if headline and not args.no_cpu_baseline:
+    progress("cpu baseline")
     line["cpu_baseline"] = run_cpu_baseline()
+  progress("done")
   print(json.dumps(line))
 
 

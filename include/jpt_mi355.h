@@ -344,7 +344,7 @@ int32_t jpt_prefill_insert_prompts(const jpt_prefill_insert_args* args,
  * The device must be the launch's own.  The streaming kernel is one
  * persistent workgroup per compute unit (all of a unit's LDS), and a slot
  * that is cut into three or more chunks is folded by a wave that waits -
- * up to a tenth of a second - for chunks that belong to OTHER workgroups of
+ * for some 60 ms at most - for chunks that belong to OTHER workgroups of
  * the same launch.  If part of the grid cannot be resident while the rest
  * runs (compute units masked off, or held for that long by a kernel of another
  * stream or process), that wait runs out and the launch gives up.  Kernels of

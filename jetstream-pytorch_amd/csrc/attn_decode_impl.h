@@ -68,7 +68,7 @@ constexpr int kSideBytes = 512;     // ks | vs | mask, 128 bytes each at most
 constexpr int kOStride = 140;       // padded LDS row of 128 outputs
 constexpr int kLdsBudget = 160 * 1024 / kGroups - 512;  // per group; one workgroup per compute unit
 constexpr int kSpinLimit = 1 << 18;  // tens of milliseconds
-constexpr uint64_t kMergeWaitTicks = 10 * 1000 * 1000;  // 0.1 s of the 100 MHz clock: a merge's wait for other workgroups' chunks
+constexpr int kMergeSpinLimit = 1 << 16;  // polls of a merge's wait for other workgroups' chunks
 // Cache policy of the loads that stream the cache (keys, values, their scales):
 // non-temporal - every byte is read once per launch, and lines kept for it in
 // the caches only push out what is read again (query rows, page ids, masks).
@@ -595,15 +595,14 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
   auto merge_item = [&](const Item& it) -> bool {
     int32_t* counter = p.arrivals + static_cast<int64_t>(it.slot) * a.kv_heads + it.h;
     // The chunks belong to other workgroups, which must get to run for this wait
-    // to end: it is sized in time (the constant 100 MHz clock), long enough for
-    // workgroups held back by other work on the device to be scheduled.
-    const uint64_t wait_from = __builtin_amdgcn_s_memrealtime();
-    for (;;) {
+    // to end: it is a long one (a poll takes about a microsecond with its sleep:
+    // some 60 ms in all), long enough for workgroups held back by other work on
+    // the device to be scheduled.
+    for (int spins = 0;; ++spins) {
       int seen = 0;
       if (lane == 0) seen = __hip_atomic_fetch_add(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (__builtin_amdgcn_readfirstlane(seen) >= it.n_chunks) break;
-      if (__builtin_amdgcn_s_memrealtime() - wait_from > kMergeWaitTicks ||
-          __hip_atomic_load(&sm_abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) {
+      if (spins > kMergeSpinLimit || __hip_atomic_load(&sm_abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) {
         give_up();
         return false;
       }

@@ -172,7 +172,7 @@ def replay_manager(w, seed, total, ps, max_pages, batch):
     om.reserve_pages_insert(slot, int(w["initial_lengths"][slot]))
   for entry in w["state"]["log"]:
     if entry[0] == "insert":
-      _, slot, n, ids = entry
+      _, slot, n, ids, _ = entry
       om.free_pages_resource(slot)
       num, view = om.reserve_pages_insert(slot, n)
       assert np.array_equal(np.asarray(view[:num]), ids)
@@ -180,7 +180,7 @@ def replay_manager(w, seed, total, ps, max_pages, batch):
       for slot in entry[1]:
         om.free_pages_resource(int(slot))
     elif entry[0] == "insert_many":
-      for slot, n, ids in zip(*entry[1:]):
+      for slot, n, ids in zip(*entry[1:4]):
         num, view = om.reserve_pages_insert(int(slot), int(n))
         assert np.array_equal(np.asarray(view[:num]), ids)
     else:
@@ -261,11 +261,11 @@ def test_c5_paged_int8_prompt_churn_and_decode_steps(host_alloc):
         continue
       if entry[0] in ("insert", "insert_many"):
         prompts = [entry[1:]] if entry[0] == "insert" else zip(*entry[1:])
-        for slot, n, ids in prompts:
+        for slot, n, ids, j in prompts:  # j: which of the step's prompt buffers
           n = int(n)
           pages = torch.from_numpy(ids.astype(np.int64)).to(dev)
           for src, wc, ws in ((w["prompts"][0], wk, wsk), (w["prompts"][1], wv, wsv)):
-            codes, sc = oquant.quantize_insert(src[l, :, :n].cpu()[None], compute_dtype=torch.float32)
+            codes, sc = oquant.quantize_insert(src[j, l, :, :n].cpu()[None], compute_dtype=torch.float32)
             padded = torch.zeros((8, len(ids) * 64, bench.D), dtype=torch.int8)
             padded[:, :n] = codes[0]
             wc[:, pages] = padded.reshape(8, len(ids), 64, bench.D).to(dev)
