@@ -495,6 +495,36 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
       else overflow();
     }
   }
+  // The order of a worker's items.  The deal gives every bin its entries longest first;
+  // a worker ends sooner when its LONGEST whole slot comes last (its many tiles keep all
+  // consumers busy to the end, the new token's tile and the change of item are long past
+  // when the last tile lands) and the short ones before it, so the whole-slot entries of
+  // a bin are rotated by one: b, ..., a, c for c >= b >= ... >= a.  (Measured on the same
+  // tensors: the headline workload's launch 34.3 -> 33.6 us.)  Chunks of cut slots keep
+  // their places: pairs must share a round, partials must be parked early.
+  if (regular) {
+    __threadfence_block();
+    __syncthreads();
+    const int rounds_used = (n_places + per_round - 1) / per_round;
+    for (int x = tid; x < per_round; x += blockDim.x) {
+      int first = -1, before = -1;
+      PlanEntry longest{};
+      for (int r = 0; r < rounds_used; ++r) {
+        const int at = r * per_round + bin_of_place(r, x);
+        if (at >= n_places) continue;
+        const PlanEntry e = entries[at];
+        if (e.slot < 0 || e.n_chunks != 1) continue;
+        if (first < 0) {
+          first = at;
+          longest = e;
+        } else {
+          entries[before] = e;  // every later whole slot moves up one
+        }
+        before = at;
+      }
+      if (first >= 0 && before != first) entries[before] = longest;
+    }
+  }
   __syncthreads();
   if (tid < kHandOutCounters) status[kStateHandOut + tid * kStateHandOutStride] = 0;
   if (tid == 0) {

@@ -7,8 +7,9 @@ groups walk in the same round, with every earlier round full; every other cut
 slot has consecutive partial records and one merge entry that names them all.
 The deal itself is pinned too: a host model of the planner's rule - entries that
 are not a pair's go, longest first, to the bin with the fewest tiles so far (or
-round the bins in snake order when that is even enough already) - must put the
-same number of tiles on every place as the plan read back from the device.
+round the bins in snake order when that is even enough already), and every bin's
+whole slots are then walked with the longest last - must put the same number of
+tiles on every place as the plan read back from the device.
 """
 import numpy as np
 import pytest
@@ -75,16 +76,26 @@ def model_deal(places, batch, kv_heads):
   max_entries = (2 * batch + 2 * extra + 3 * (w // kv_heads + 8) + 7) // 8 * 8
   max_rounds = max((max_entries - batch) // per_round, 1)
   cap = max(max_rounds - (len(others) - one_by_one + per_round - 1) // per_round, 1)
-  for _, t in others[:one_by_one]:
+  whole = [False] * len(places)  # places that hold a whole slot (not a chunk of a cut one)
+  for kind, t in others[:one_by_one]:
     x = min((b for b in range(per_round) if rounds[b] < cap), key=lambda b: (load[b], b))
-    out[rounds[x] * per_round + bin_of(rounds[x], x)] = t
+    at = rounds[x] * per_round + bin_of(rounds[x], x)
+    out[at], whole[at] = t, kind == 0
     load[x] += t
     rounds[x] += 1
-  for i, (_, t) in enumerate(others[one_by_one:]):
+  for i, (kind, t) in enumerate(others[one_by_one:]):
     lap, x = divmod(i, per_round)
     x = per_round - 1 - x if lap & 1 else x
     rnd = rounds[x] + lap
-    out[rnd * per_round + bin_of(rnd, x)] = t
+    at = rnd * per_round + bin_of(rnd, x)
+    out[at], whole[at] = t, kind == 0
+  # the whole slots of a bin, dealt longest first, are walked with the longest last
+  for x in range(per_round):
+    mine = [rnd * per_round + bin_of(rnd, x) for rnd in range((len(places) + per_round - 1) // per_round)]
+    mine = [at for at in mine if at < len(places) and whole[at]]
+    tiles = [out[at] for at in mine]
+    for at, t in zip(mine, tiles[1:] + tiles[:1]):
+      out[at] = t
   return out
 
 
