@@ -15,6 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 OUT_DIR = os.path.join(HERE, "jetstream_pt_amd")
 LIB = os.path.join(OUT_DIR, "libjpt_mi355.so")
+TIMELINE_LIB = os.path.join(OUT_DIR, "libjpt_mi355_timeline.so")
 BUILD = os.path.join(HERE, "build")
 
 SOURCES = ["api.cpp", "pam.cpp", "kv_lines.hip", "prefill_insert.hip", "paged_kv.hip", "device_pages.hip", "attn_generic.hip", "attn_decode.hip",
@@ -29,9 +30,9 @@ FLAGS = [
 ]
 
 
-def _compile(src):
-  obj = os.path.join(BUILD, os.path.splitext(src)[0] + ".o")
-  cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(src, extra=(), tag=""):
+  obj = os.path.join(BUILD, os.path.splitext(src)[0] + tag + ".o")
+  cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
   r = subprocess.run(cmd, capture_output=True, text=True)
   # the host pass does not know the device-only target feature; drop its note
   err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
@@ -42,18 +43,34 @@ def _compile(src):
   return obj
 
 
-def build(verbose=True):
-  os.makedirs(BUILD, exist_ok=True)
-  with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as ex:
-    objs = list(ex.map(_compile, SOURCES))
-  tmp = LIB + ".tmp"
+def _link(objs, lib):
+  tmp = lib + ".tmp"
   cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]
   r = subprocess.run(cmd, capture_output=True, text=True)
   if r.returncode != 0:
     raise RuntimeError(f"link failed:\n{r.stderr}")
-  os.replace(tmp, LIB)
+  os.replace(tmp, lib)
+
+
+def build(verbose=True, timeline=True):
+  """The product library, and (timeline) its development twin libjpt_mi355_timeline.so, whose
+  decode-attention kernel records when its waves start, stream and end (attn_timeline.py);
+  nothing of the package loads the twin unless JPT_MI355_LIB names it."""
+  os.makedirs(BUILD, exist_ok=True)
+  traced = ["attn_decode_i8.hip", "attn_decode_bf16.hip"]  # the units that hold the streaming kernel
+  with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as ex:
+    plain = [ex.submit(_compile, src) for src in SOURCES]
+    twin = [ex.submit(_compile, src, ("-DJPT_ATTN_TIMELINE",), "_timeline") for src in traced] if timeline else []
+    objs = [f.result() for f in plain]
+    twin = [f.result() for f in twin]
+  _link(objs, LIB)
   if verbose:
     print(f"built {LIB}")
+  if timeline:
+    swapped = [o for o, src in zip(objs, SOURCES) if src not in traced] + twin
+    _link(swapped, TIMELINE_LIB)
+    if verbose:
+      print(f"built {TIMELINE_LIB}")
   return LIB
 
 

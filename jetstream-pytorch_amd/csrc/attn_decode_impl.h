@@ -47,6 +47,17 @@
 #include "attn_common.h"
 #include "attn_plan.h"
 
+// Development aid, off in the product library: with JPT_ATTN_TIMELINE defined every wave of
+// the first 256 workgroups leaves four words in the workspace's state block (from byte 1024:
+// [workgroup][group][producer, consumers 0..2][start, first tile, end, tiles | items << 16],
+// times on the constant 100 MHz clock), from which attn_timeline.py derives when workers
+// start, stream and end.  build_lib.py --timeline builds that library beside the product's.
+#ifdef JPT_ATTN_TIMELINE
+#define JPT_TL(...) __VA_ARGS__
+#else
+#define JPT_TL(...)
+#endif
+
 namespace jpt {
 namespace decode {
 
@@ -414,6 +425,17 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
   if (tid < kGroups * C::kQBufs) (&sm_qtaken_all[0][0])[tid] = 0;
 
   if (tid == 0) sm_abort = 0;
+  JPT_TL(
+  int* const tl_rec = reinterpret_cast<int*>(reinterpret_cast<char*>(p.status) + 1024) +
+      ((static_cast<int>(blockIdx.x) * kGroups + group) * 4 + (wave == kConsumers ? 0 : wave + 1)) * 4;
+  const int tl_start = static_cast<int>(__builtin_amdgcn_s_memrealtime());
+  int tl_first = 0, tl_tiles = 0, tl_items = 0;
+  auto tl_now = [] { return static_cast<int>(__builtin_amdgcn_s_memrealtime()); };
+  auto tl_write = [&]() {
+    if (lane == 0 && blockIdx.x < 256) {
+      tl_rec[0] = tl_start; tl_rec[1] = tl_first; tl_rec[2] = tl_now(); tl_rec[3] = tl_tiles | (tl_items << 16);
+    }
+  };)
 
   const int R = p.rows;
   // The groups of all workgroups are the workers; worker ids of one workgroup
@@ -850,6 +872,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
         if (lane < kTile) __builtin_amdgcn_global_load_lds((global_ptr)(mk + lane), (lds_ptr)(side + 256), 4, 0, 0);
       }
       ++issued;
+      JPT_TL(if (tl_first == 0) tl_first = tl_now(); ++tl_tiles;)
       loads_issued += C::kLoadsPerTile;
       if (++fill_slot == C::kSlots) { fill_slot = 0; ++fill_round; }
       return true;
@@ -976,6 +999,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
       }
       __builtin_amdgcn_s_sleep(1);
     }
+    JPT_TL(tl_write();)
     // Every tile of this worker has landed; its consumers are working off the
     // ring.  The producer now folds split slots: it takes (merge entry, head)
     // pairs from a counter in memory for as long as there are any - the workers
@@ -1144,6 +1168,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
     if (!wait_for(&sm_filled[s], t / C::kSlots + 1)) return false;
     char* slot = ring + s * C::kSlotBytes;
     const char* side = slot + 2 * C::kTileBytes;
+    JPT_TL(if (tl_first == 0) tl_first = tl_now(); ++tl_tiles;)
     float new_ks = 0.f, new_vs = 0.f;
     const bool quant_here = is_new && quant_new;
     if (quant_here) {
@@ -1439,10 +1464,12 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
         }
       }
     }
+    JPT_TL(++tl_items;)
     if (!finish_item(cur, seq++)) return;
     base += nt;
   }
   count_parked_chunk();
+  JPT_TL(tl_write();)
 }
 
 // `workers` groups are wanted; a workgroup holds kGroups of them.
