@@ -424,10 +424,21 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     // bin of the plain snake deal over the sorted list is within 1/32 of the mean
     // (batches of similar lengths), the snake it is.
     if (candidates > 0) {
+      // (one atomic a wave: a hundred of them on one LDS word took 4 us)
+      int heaviest = 0, sum = 0;
       for (int x = tid; x < per_round; x += blockDim.x) {
         const int load = s_bin_load[x] + s_snake_load[x];
-        atomicMax(&s_snake_max, load);
-        atomicAdd(&s_snake_sum, load);
+        heaviest = max(heaviest, load);
+        sum += load;
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        heaviest = max(heaviest, __shfl_xor(heaviest, off));
+        sum += __shfl_xor(sum, off);
+      }
+      if ((tid & 63) == 0) {
+        atomicMax(&s_snake_max, heaviest);
+        atomicAdd(&s_snake_sum, sum);
       }
       __syncthreads();
     }
@@ -458,6 +469,7 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
     const int round = s_bin_rounds[x] + lap;  // one entry a bin and lap
     return round * per_round + bin_of_place(round, x);
   };
+  int last_place = 0;  // one past the last place this thread wrote
   for (int b = tid; b < batch; b += blockDim.x) {
     const int nc = chunks_of(b), cl = chunk_len(b), first = s_first[b];
     if (paired(b)) {
@@ -467,7 +479,7 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
       if (at + half < max_entries) {
         entries[at] = PlanEntry{b, 0, cl, -1, 2, s_len[b], {0, 0}};
         entries[at + half] = PlanEntry{b, cl, s_len[b] - cl, -1, 2, s_len[b], {0, 0}};
-        atomicMax(&s_positions, at + half + 1);
+        last_place = max(last_place, at + half + 1);
       } else {
         overflow();
       }
@@ -478,12 +490,15 @@ plan_kernel(const int32_t* lengths, int batch, int seq_cap, int kv_heads, int ta
       const int at = place_of(atomicAdd(&s_base[key_of(count, nc > 1 ? 1 : 0)], 1) - n_pairs);
       if (at < max_entries) {
         entries[at] = PlanEntry{b, c * cl, count, first + c, nc, s_len[b], {0, 0}};
-        atomicMax(&s_positions, at + 1);
+        last_place = max(last_place, at + 1);
       } else {
         overflow();
       }
     }
   }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) last_place = max(last_place, __shfl_xor(last_place, off));
+  if ((tid & 63) == 0) atomicMax(&s_positions, last_place);
   __syncthreads();
   // merge entries, one for every slot cut in three or more (or in two where there is no pairing), after the last place
   const int n_places = min(s_positions, max_entries);
