@@ -9,7 +9,7 @@ a summary: first load, first tile consumed, the producers' last tile, the
 groups' ends, and a least-squares fit of a bin's end time on its tiles and items
 (a bin = the eight workers that take the heads of one plan entry).
 
-  python jetstream-pytorch_amd/attn_timeline.py [--case c3|<positions per slot>] [--unfused]
+  python jetstream-pytorch_amd/attn_timeline.py [--case c3|<positions per slot>|uniform:LO:HI] [--batch B] [--unfused]
 
 Times are in microseconds from the first wave's start, on the constant 100 MHz
 clock; the kernel's duration by the host's clock is about 1.8 us longer than the
@@ -37,12 +37,16 @@ from jetstream_pt_amd import attention_kernel as ak  # noqa: E402
 
 def main():
   ap = argparse.ArgumentParser()
-  ap.add_argument("--case", default="c3", help="c3, or a number: every slot that many positions long")
+  ap.add_argument("--case", default="c3", help="c3; a number: every slot that many positions long; "
+                  "uniform:LO:HI: lengths drawn uniformly from [LO, HI] (seed 4)")
+  ap.add_argument("--batch", type=int, default=0, help="slots (default: the headline workload's 128)")
   ap.add_argument("--unfused", action="store_true", help="attention over the cache only, no new token")
   ap.add_argument("--reps", type=int, default=3)
   args = ap.parse_args()
   dev = "cuda"
-  b, hq, hkv, s, d, nl = bench.B, bench.HQ, bench.HKV, bench.S, bench.D, 8
+  b, hq, hkv, s, d, nl = args.batch or bench.B, bench.HQ, bench.HKV, bench.S, bench.D, 8
+  if b > bench.B:
+    s, nl = s * bench.B // b, 4  # the same bytes of cache
   torch.manual_seed(3)
   k = torch.empty((nl, b, hkv, s, d), dtype=torch.int8, device=dev)
   v = torch.empty_like(k)
@@ -58,7 +62,13 @@ def main():
   nv = torch.zeros_like(nk)
   nks = torch.zeros((b, 1, 1, 1), device=dev)
   nvs = torch.zeros_like(nks)
-  lengths = bench.seeded_lengths(torch) if args.case == "c3" else torch.full((b,), int(args.case))
+  if args.case == "c3":
+    lengths = bench.seeded_lengths(torch, b)
+  elif args.case.startswith("uniform:"):
+    lo, hi = (int(x) for x in args.case.split(":")[1:])
+    lengths = bench.uniform_lengths(torch, b, lo, min(hi, s - 1), 4)
+  else:
+    lengths = torch.full((b,), int(args.case))
   lengths = lengths.to(dev).to(torch.int32)
   plan, _ = ak.precompute_ragged_block_indices(lengths, b, hq, hkv, s)
   new = {} if args.unfused else dict(new_key=nk, new_value=nv, new_k_scaler=nks, new_v_scaler=nvs,
@@ -108,7 +118,10 @@ def main():
           % (bm.mean(), bm.std(), within.mean()))
     print("  fit over the 64 bins: end = %.3f * tiles + %.2f * items + %.2f, residual std %.2f"
           % (coef[0], coef[1], coef[2], (bm - a @ coef).std()))
-    print("  per XCD, mean end: " + " ".join("%.1f" % gend[np.arange(256) % 8 == x].mean() for x in range(8)))
+    xcd = np.arange(256) % 8
+    print("  per XCD, mean end: " + " ".join("%.1f" % gend[xcd == x].mean() for x in range(8)))
+    print("  per XCD, producers' first load: " + " ".join("%.2f" % us(prod[..., 1])[xcd == x].mean() for x in range(8))
+          + "; last tile landed: " + " ".join("%.1f" % us(prod[..., 2])[xcd == x].mean() for x in range(8)))
 
 
 if __name__ == "__main__":
