@@ -21,8 +21,9 @@ def kats():
 
 
 # Largest absolute attention-output error each GPU parity check saw, with the
-# largest magnitude of the expected values beside it; written under gpurun_out/
-# at the end of a GPU session (the figures DESIGN.md quotes come from there).
+# largest magnitude of the expected values beside it; written as
+# parity_max_abs.json into the run's output folder at the end of a GPU session
+# (the measured errors the documentation quotes come from there).
 PARITY_ERRORS = {}
 
 
