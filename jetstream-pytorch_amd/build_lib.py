@@ -18,8 +18,11 @@ LIB = os.path.join(OUT_DIR, "libjpt_mi355.so")
 TIMELINE_LIB = os.path.join(OUT_DIR, "libjpt_mi355_timeline.so")
 BUILD = os.path.join(HERE, "build")
 
-SOURCES = ["api.cpp", "pam.cpp", "kv_lines.hip", "prefill_insert.hip", "paged_kv.hip", "device_pages.hip", "attn_generic.hip", "attn_decode.hip",
-           "attn_decode_i8.hip", "attn_decode_bf16.hip"]
+# the units that hold the streaming attention kernel, one per cache type and way the new token comes
+STREAMING = ["attn_decode_i8_raw.hip", "attn_decode_i8_raw_wide.hip", "attn_decode_i8_raw_rope.hip", "attn_decode_i8_raw_wide_rope.hip",
+             "attn_decode_i8_none.hip", "attn_decode_i8_given.hip", "attn_decode_bf16_given.hip", "attn_decode_bf16_none.hip"]
+SOURCES = STREAMING + ["api.cpp", "pam.cpp", "kv_lines.hip", "prefill_insert.hip", "paged_kv.hip", "device_pages.hip", "attn_generic.hip",
+                       "attn_decode.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -57,7 +60,7 @@ def build(verbose=True, timeline=True):
   decode-attention kernel records when its waves start, stream and end (attn_timeline.py);
   nothing of the package loads the twin unless JPT_MI355_LIB names it."""
   os.makedirs(BUILD, exist_ok=True)
-  traced = ["attn_decode_i8.hip", "attn_decode_bf16.hip"]  # the units that hold the streaming kernel
+  traced = STREAMING
   with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as ex:
     plain = [ex.submit(_compile, src) for src in SOURCES]
     twin = [ex.submit(_compile, src, ("-DJPT_ATTN_TIMELINE",), "_timeline") for src in traced] if timeline else []

@@ -622,8 +622,18 @@ int32_t attn_fast_launch(const jpt_attn_args& a, AttnMode mode, hipStream_t stre
   }
   int32_t blocks = persistent_blocks();
   if (blocks > p.total_items) blocks = p.total_items;  // total_items is a multiple of 8
-  if (a.kv_dtype == JPT_I8) decode::launch_decode_i8(p, mode == kPaged, blocks, stream);
-  else decode::launch_decode_bf16(p, mode == kPaged, blocks, stream);
+  const bool paged = mode == kPaged;
+  if (a.kv_dtype == JPT_I8) {
+    if (!a.new_k) decode::launch_decode_i8_none(p, paged, blocks, stream);
+    else if (!a.new_k_raw) decode::launch_decode_i8_given(p, paged, blocks, stream);
+    else if (a.kv_heads <= 16 && !a.new_k_rope) decode::launch_decode_i8_raw(p, paged, blocks, stream);
+    else if (a.kv_heads <= 16) decode::launch_decode_i8_raw_rope(p, paged, blocks, stream);
+    else if (!a.new_k_rope) decode::launch_decode_i8_raw_wide(p, paged, blocks, stream);
+    else decode::launch_decode_i8_raw_wide_rope(p, paged, blocks, stream);
+  } else {
+    if (!a.new_k) decode::launch_decode_bf16_none(p, paged, blocks, stream);
+    else decode::launch_decode_bf16_given(p, paged, blocks, stream);
+  }
   return launch_status("attn_decode_kernel");
 }
 

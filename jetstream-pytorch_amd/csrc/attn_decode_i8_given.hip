@@ -1,0 +1,10 @@
+// int8-KV instantiations of the streaming decode attention kernel: new token given as the cache holds it.
+#include "attn_decode_impl.h"
+
+namespace jpt {
+namespace decode {
+void launch_decode_i8_given(const FastParams& p, bool paged, unsigned blocks, hipStream_t stream) {
+  launch_decode<int8_t, kNewGiven>(p, paged, blocks, stream);
+}
+}  // namespace decode
+}  // namespace jpt

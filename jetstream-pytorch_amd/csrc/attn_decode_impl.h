@@ -367,7 +367,11 @@ struct Item {
   __device__ __forceinline__ bool merge() const { return start < 0; }
 };
 
-template <typename KV, bool PAGED, int SCALE, bool MASK, int RC>
+// NEW: how the step's new token comes (kNew*): compile-time, because each of these few
+// branches in the producer's and the consumers' loops costs scalar registers and code the
+// common launch never runs (the headline workload's launch 33.05 -> 32.5 us on the same
+// tensors when they became constants).
+template <typename KV, bool PAGED, int SCALE, bool MASK, int RC, int NEW>
 __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(FastParams p) {
   using C = Config<KV, SCALE, MASK, RC>;
   const jpt_attn_args& a = p.a;
@@ -458,12 +462,13 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
   }
   const int n_ids = (n_entries + 7) / 8 * 8 * a.kv_heads;  // item ids that may name a work entry
   const int n_rounds = (n_ids + G - 1) / G;
-  const bool has_new = a.new_k != nullptr;
+  constexpr bool has_new = NEW != kNewNone;
   // the new token arrives unquantised: the consumer of its tile quantises it
-  const bool quant_new = std::is_same<KV, int8_t>::value && a.new_k_raw != nullptr;
+  constexpr bool quant_new = std::is_same<KV, int8_t>::value && NEW >= kNewRaw;
   // more than 16 KV heads: the token's raw rows fill two tiles, keys then values,
   // each spread over the key and the value area; one consumer takes both
-  const bool wide_new = quant_new && a.kv_heads > 16;
+  constexpr bool wide_new = quant_new && (NEW == kNewRawWide || NEW == kNewRawWideRope);
+  constexpr bool rope_new = quant_new && (NEW == kNewRawRope || NEW == kNewRawWideRope);  // the key is rotated first
   // the new token is also written into its slot's page (paged caches)
   const bool to_pages = PAGED && has_new && a.new_to_pages != 0;
 
@@ -1172,7 +1177,7 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
     float new_ks = 0.f, new_vs = 0.f;
     const bool quant_here = is_new && quant_new;
     if (quant_here) {
-      const float* rope = a.new_k_rope ? a.new_k_rope + static_cast<int64_t>(cur_slot) * kD : nullptr;
+      const float* rope = rope_new ? a.new_k_rope + static_cast<int64_t>(cur_slot) * kD : nullptr;
       float k0, k1, v0, v1;
       // the raw value rows: this tile's value area, or all of the next tile
       const char* v_rows = slot + C::kTileBytes;
@@ -1473,34 +1478,36 @@ __global__ void __launch_bounds__(kThreads, kWavesPerSimd) attn_decode_kernel(Fa
 }
 
 // `workers` groups are wanted; a workgroup holds kGroups of them.
-template <typename KV, bool PAGED, int SCALE, bool MASK>
+template <typename KV, bool PAGED, int SCALE, bool MASK, int NEW>
 void launch_rows(const FastParams& p, unsigned workers, hipStream_t stream) {
   const unsigned blocks = workers / kGroups > 0 ? workers / kGroups : 1;
   if (p.rows <= 4)
-    hipLaunchKernelGGL((attn_decode_kernel<KV, PAGED, SCALE, MASK, 4>), dim3(blocks), dim3(kThreads), 0, stream, p);
+    hipLaunchKernelGGL((attn_decode_kernel<KV, PAGED, SCALE, MASK, 4, NEW>), dim3(blocks), dim3(kThreads), 0, stream, p);
   else if (p.rows <= 8)
-    hipLaunchKernelGGL((attn_decode_kernel<KV, PAGED, SCALE, MASK, 8>), dim3(blocks), dim3(kThreads), 0, stream, p);
+    hipLaunchKernelGGL((attn_decode_kernel<KV, PAGED, SCALE, MASK, 8, NEW>), dim3(blocks), dim3(kThreads), 0, stream, p);
   else
-    hipLaunchKernelGGL((attn_decode_kernel<KV, PAGED, SCALE, MASK, 16>), dim3(blocks), dim3(kThreads), 0, stream, p);
+    hipLaunchKernelGGL((attn_decode_kernel<KV, PAGED, SCALE, MASK, 16, NEW>), dim3(blocks), dim3(kThreads), 0, stream, p);
 }
 
-template <typename KV, bool PAGED, int SCALE>
+template <typename KV, bool PAGED, int SCALE, int NEW>
 void launch_masked(const FastParams& p, unsigned blocks, hipStream_t stream) {
-  if (!PAGED && p.a.mask) launch_rows<KV, PAGED, SCALE, !PAGED>(p, blocks, stream);
-  else launch_rows<KV, PAGED, SCALE, false>(p, blocks, stream);
+  if (!PAGED && p.a.mask) launch_rows<KV, PAGED, SCALE, !PAGED, NEW>(p, blocks, stream);
+  else launch_rows<KV, PAGED, SCALE, false, NEW>(p, blocks, stream);
 }
 
-template <typename KV>
+// One translation unit per (cache type, NEW) instantiates this: the kernels of one unit take
+// about a minute to compile, and the units compile side by side.
+template <typename KV, int NEW>
 void launch_decode(const FastParams& p, bool paged, unsigned blocks, hipStream_t stream) {
   const int scale = !p.a.k_scale ? kNoScale : p.a.scale_dtype == JPT_F32 ? kScaleF32 : kScaleBF16;
   if (paged) {
-    if (scale == kNoScale) launch_masked<KV, true, kNoScale>(p, blocks, stream);
-    else if (scale == kScaleF32) launch_masked<KV, true, kScaleF32>(p, blocks, stream);
-    else launch_masked<KV, true, kScaleBF16>(p, blocks, stream);
+    if (scale == kNoScale) launch_masked<KV, true, kNoScale, NEW>(p, blocks, stream);
+    else if (scale == kScaleF32) launch_masked<KV, true, kScaleF32, NEW>(p, blocks, stream);
+    else launch_masked<KV, true, kScaleBF16, NEW>(p, blocks, stream);
   } else {
-    if (scale == kNoScale) launch_masked<KV, false, kNoScale>(p, blocks, stream);
-    else if (scale == kScaleF32) launch_masked<KV, false, kScaleF32>(p, blocks, stream);
-    else launch_masked<KV, false, kScaleBF16>(p, blocks, stream);
+    if (scale == kNoScale) launch_masked<KV, false, kNoScale, NEW>(p, blocks, stream);
+    else if (scale == kScaleF32) launch_masked<KV, false, kScaleF32, NEW>(p, blocks, stream);
+    else launch_masked<KV, false, kScaleBF16, NEW>(p, blocks, stream);
   }
 }
 

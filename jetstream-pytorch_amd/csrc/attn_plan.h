@@ -46,10 +46,24 @@ struct FastParams {
   int32_t* status;      // the workspace's state block (kState* words)
 };
 
+// How the step's new token reaches the streaming kernel (a template argument of it).
+constexpr int kNewNone = 0;     // no new token: the cache only
+constexpr int kNewGiven = 1;    // rows as the cache holds them (bf16, or codes with their scales)
+constexpr int kNewRaw = 2;      // int8 caches: unquantised rows of all heads in one tile, quantised in the launch
+constexpr int kNewRawWide = 3;  // the same with more than 16 KV heads: two tiles, keys then values
+constexpr int kNewRawRope = 4;      // kNewRaw, the key rotated (rotary embedding) before it is quantised
+constexpr int kNewRawWideRope = 5;  // kNewRawWide, likewise
+
 namespace decode {
-// Defined in attn_decode_i8.hip / attn_decode_bf16.hip.
-void launch_decode_i8(const FastParams& p, bool paged, unsigned blocks, hipStream_t stream);
-void launch_decode_bf16(const FastParams& p, bool paged, unsigned blocks, hipStream_t stream);
+// Defined in attn_decode_i8_new<N>.hip / attn_decode_bf16_new<N>.hip, one unit per way the new token comes.
+void launch_decode_i8_none(const FastParams& p, bool paged, unsigned blocks, hipStream_t stream);
+void launch_decode_i8_given(const FastParams& p, bool paged, unsigned blocks, hipStream_t stream);
+void launch_decode_i8_raw(const FastParams& p, bool paged, unsigned blocks, hipStream_t stream);
+void launch_decode_i8_raw_wide(const FastParams& p, bool paged, unsigned blocks, hipStream_t stream);
+void launch_decode_i8_raw_rope(const FastParams& p, bool paged, unsigned blocks, hipStream_t stream);
+void launch_decode_i8_raw_wide_rope(const FastParams& p, bool paged, unsigned blocks, hipStream_t stream);
+void launch_decode_bf16_none(const FastParams& p, bool paged, unsigned blocks, hipStream_t stream);
+void launch_decode_bf16_given(const FastParams& p, bool paged, unsigned blocks, hipStream_t stream);
 }  // namespace decode
 
 }  // namespace jpt
