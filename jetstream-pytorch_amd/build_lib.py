@@ -60,7 +60,8 @@ def build(verbose=True, timeline=True):
   decode-attention kernel records when its waves start, stream and end (attn_timeline.py);
   nothing of the package loads the twin unless JPT_MI355_LIB names it."""
   os.makedirs(BUILD, exist_ok=True)
-  traced = STREAMING
+  # the twin's own units: what attn_timeline.py launches (int8 cache, raw token or none); the rest are the product's
+  traced = ["attn_decode_i8_raw.hip", "attn_decode_i8_none.hip"]
   with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as ex:
     plain = [ex.submit(_compile, src) for src in SOURCES]
     twin = [ex.submit(_compile, src, ("-DJPT_ATTN_TIMELINE",), "_timeline") for src in traced] if timeline else []

@@ -565,6 +565,8 @@ bool attn_fast_supported(const jpt_attn_args& a, AttnMode mode) {
                  a.mask_stride_b % 4 != 0 || !aligned(a.mask, 16)))
     return false;
   if (a.k_scale && (!aligned(a.k_scale, 16) || !aligned(a.v_scale, 16))) return false;
+  // the streaming kernel is built for the caches the path has: int8 codes with scales, bf16 without
+  if ((a.kv_dtype == JPT_I8) != (a.k_scale != nullptr)) return false;
   if (!aligned(a.q, 16) || !aligned(a.k, 16) || !aligned(a.v, 16)) return false;
   if (a.new_k && (!aligned(a.new_k, 16) || !aligned(a.new_v, 16))) return false;
   // the new token's raw rows of all heads must fit a tile (its key and value areas together)

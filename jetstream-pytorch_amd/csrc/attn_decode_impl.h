@@ -1496,18 +1496,22 @@ void launch_masked(const FastParams& p, unsigned blocks, hipStream_t stream) {
 }
 
 // One translation unit per (cache type, NEW) instantiates this: the kernels of one unit take
-// about a minute to compile, and the units compile side by side.
+// about a minute to compile, and the units compile side by side.  int8 caches come with scales
+// (float32 or bf16), bf16 caches without: nothing else is built (attn_fast_supported).
 template <typename KV, int NEW>
 void launch_decode(const FastParams& p, bool paged, unsigned blocks, hipStream_t stream) {
-  const int scale = !p.a.k_scale ? kNoScale : p.a.scale_dtype == JPT_F32 ? kScaleF32 : kScaleBF16;
-  if (paged) {
-    if (scale == kNoScale) launch_masked<KV, true, kNoScale, NEW>(p, blocks, stream);
-    else if (scale == kScaleF32) launch_masked<KV, true, kScaleF32, NEW>(p, blocks, stream);
-    else launch_masked<KV, true, kScaleBF16, NEW>(p, blocks, stream);
+  if constexpr (std::is_same<KV, int8_t>::value) {
+    const bool f32 = p.a.scale_dtype == JPT_F32;
+    if (paged) {
+      if (f32) launch_masked<KV, true, kScaleF32, NEW>(p, blocks, stream);
+      else launch_masked<KV, true, kScaleBF16, NEW>(p, blocks, stream);
+    } else {
+      if (f32) launch_masked<KV, false, kScaleF32, NEW>(p, blocks, stream);
+      else launch_masked<KV, false, kScaleBF16, NEW>(p, blocks, stream);
+    }
   } else {
-    if (scale == kNoScale) launch_masked<KV, false, kNoScale, NEW>(p, blocks, stream);
-    else if (scale == kScaleF32) launch_masked<KV, false, kScaleF32, NEW>(p, blocks, stream);
-    else launch_masked<KV, false, kScaleBF16, NEW>(p, blocks, stream);
+    if (paged) launch_masked<KV, true, kNoScale, NEW>(p, blocks, stream);
+    else launch_masked<KV, false, kNoScale, NEW>(p, blocks, stream);
   }
 }
 
