@@ -3,13 +3,14 @@ kernel trusts the planner's records (it never checks one), so the properties
 it relies on are checked here on the planner's own output: whatever the
 lengths, the work entries cover every position of every slot exactly once;
 the two chunks of a slot cut in two sit on places that one workgroup's two
-groups walk in the same round, with every earlier round full; every other cut
-slot has consecutive partial records and one merge entry that names them all.
-The deal itself is pinned too: a host model of the planner's rule - entries that
-are not a pair's go, longest first, to the bin with the fewest tiles so far (or
-round the bins in snake order when that is even enough already), and every bin's
-whole slots are then walked with the longest last - must put the same number of
-tiles on every place as the plan read back from the device.
+groups walk in the same round, with an item of both on every earlier round; every
+other cut slot has consecutive partial records and one merge entry that names them
+all.  The deal itself is pinned too: a host model of the planner's rule - entries
+that are not a pair's go, longest first, to the bin with the fewest tiles so far (or
+round the bins in snake order when that is even enough already), every bin's whole
+slots are then walked with the longest last, and a workgroup's pair goes behind
+its two bins' whole slots where both hold equally many and nothing else - must put
+the same number of tiles on every place as the plan read back from the device.
 """
 import numpy as np
 import pytest
@@ -53,15 +54,23 @@ def model_deal(places, batch, kv_heads):
   bin_of = lambda rnd, x: per_round - 1 - x if rnd & 1 else x
   load, rounds = [0] * per_round, [0] * per_round
   out = [-1] * len(places)
-  n_pairs = 0
-  for at, e in enumerate(places):
-    if is_pair(e):
-      rnd, x = divmod(at, per_round)
-      first = e if x < half else places[at - half]  # both bins are charged the first chunk's tiles
-      load[bin_of(rnd, x)] += tiles_of(first[2])
-      rounds[bin_of(rnd, x)] = max(rounds[bin_of(rnd, x)], rnd + 1)
-      out[at] = tiles_of(e[2])
-      n_pairs += x < half
+  # pairs: found where the plan has them, which is where the deal put them - round by round from
+  # the first - unless the last pass moved them behind their bins' whole slots (one round of pairs
+  # only: then they were dealt to round 0)
+  members = [(at, e) for at, e in enumerate(places) if is_pair(e)]
+  n_pairs = len(members) // 2
+  pair_of_bin = {}
+  for at, e in members:
+    rnd, x = divmod(at, per_round)
+    b = bin_of(rnd, x)
+    if n_pairs <= half:
+      rnd = 0
+    partner = next(e2 for _, e2 in members if e2[0] == e[0] and e2[1] != e[1])
+    first = e if e[1] == 0 else partner  # both bins are charged the first chunk's tiles
+    load[b] += tiles_of(first[2])
+    rounds[b] = max(rounds[b], rnd + 1)
+    out[rnd * per_round + bin_of(rnd, b)] = tiles_of(e[2])
+    pair_of_bin[b] = e[0]
   if n_pairs:
     rounds = [max(r, n_pairs // half) for r in rounds]
   others = sorted(((1 if e[4] > 1 else 0, tiles_of(e[2])) for e in places if e[0] >= 0 and not is_pair(e)), reverse=True)
@@ -96,6 +105,26 @@ def model_deal(places, batch, kv_heads):
     tiles = [out[at] for at in mine]
     for at, t in zip(mine, tiles[1:] + tiles[:1]):
       out[at] = t
+  # a workgroup's two bins that hold a paired chunk each and then equally many whole slots, nothing
+  # else: the pair goes last in both, the whole slots before it shortest first
+  n_rounds = (len(places) + per_round - 1) // per_round
+  if 0 < n_pairs <= half <= 32 and n_rounds - 1 <= 8:  # (the planner stages eight rounds behind the pair's, for 32 pairs of bins)
+    for x in range(half):
+      y = x + half
+      if x not in pair_of_bin or pair_of_bin.get(y) != pair_of_bin[x]:
+        continue
+      walk = lambda b: [r * per_round + bin_of(r, b) for r in range(n_rounds) if r * per_round + bin_of(r, b) < len(places)]
+      wx, wy = walk(x), walk(y)
+      held = lambda w: [r for r, at in enumerate(w) if out[at] >= 0]
+      hx, hy = held(wx), held(wy)
+      m = len(hx) - 1
+      if hx != hy or hx != list(range(m + 1)) or not 1 <= m <= 8 or not all(whole[at] for w in (wx, wy) for at in w[1:m + 1]):
+        continue
+      for w in (wx, wy):
+        pair_tiles, tiles = out[w[0]], [out[at] for at in w[1:m + 1]]
+        new = [tiles[m - 1] if r == m - 1 else tiles[m - 2 - r] for r in range(m)] + [pair_tiles]
+        for at, t in zip(w[:m + 1], new):
+          out[at] = t
   return out
 
 
@@ -138,9 +167,13 @@ def check_plan(lengths, kv_heads, seq):
       n_pairs += 1
       (s0, c0, p0, _, at0), (s1, c1, p1, _, at1) = cs
       assert p0 == -1 and p1 == -1 and slot not in merge_of
-      assert at1 == at0 + per_round // 2 and at0 % per_round < per_round // 2
-      # the item has the same number in both groups' walks: every place of the rounds before is taken
-      assert np.all(places[:at0 // per_round * per_round, 0] >= 0)
+      bin_of = lambda at: at % per_round if (at // per_round) % 2 == 0 else per_round - 1 - at % per_round
+      rnd, b0, b1 = at0 // per_round, bin_of(at0), bin_of(at1)
+      assert at1 // per_round == rnd and abs(b1 - b0) == per_round // 2  # the two groups of one workgroup
+      # the item has the same number in both groups' walks: both bins have an item on every round before
+      for b in (b0, b1):
+        for r in range(rnd):
+          assert places[r * per_round + (b if r % 2 == 0 else per_round - 1 - b), 0] >= 0
       continue
     part0, n = merge_of[slot]
     assert n == len(cs)
